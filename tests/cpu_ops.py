@@ -209,35 +209,133 @@ class CpuOps:
     def pack_experts(self, w_gate_up, w_down):
         return None
 
-    def route_experts(self, z, experts, top, groups, keep, scale, has_shared, transposed=False):
+    def check_router(self, score, group_score):
+        assert score in ("sigmoid", "softmax") and group_score in ("top2", "max")
+
+    def route_experts(self, z, experts, top, groups, keep, scale, has_shared, transposed=False, score="sigmoid",
+                      group_score="top2", normalize=True, correction=None):
         z = z.t() if transposed else z
         T = z.shape[0]
-        s = torch.sigmoid(z[:, :experts])
+        s = torch.sigmoid(z[:, :experts]) if score == "sigmoid" else torch.softmax(z[:, :experts], dim=-1)
+        c = s if correction is None else s + correction
         per = experts // groups
-        score = s.reshape(T, groups, per).topk(min(2, per), dim=-1).values.sum(-1)
-        best = score.topk(keep, dim=-1).indices
+        by_group = c.reshape(T, groups, per)
+        group = by_group.topk(min(2, per), dim=-1).values.sum(-1) if group_score == "top2" else by_group.max(-1).values
+        best = group.topk(keep, dim=-1).indices
         open_ = torch.zeros(T, groups, dtype=torch.bool)
         open_.scatter_(1, best, True)
-        masked = torch.where(open_.repeat_interleave(per, 1), s, torch.full_like(s, -1.0))
+        masked = torch.where(open_.repeat_interleave(per, 1), c, torch.full_like(c, float("-inf")))
         ids = masked.topk(top, dim=-1).indices
         w = s.gather(1, ids)
-        w = w / (w.sum(-1, keepdim=True) + 1e-20) * scale
+        w = w / (w.sum(-1, keepdim=True) + 1e-20) * scale if normalize else w * scale
         return ids.to(torch.int32), w, (torch.sigmoid(z[:, experts]) if has_shared else None)
 
     def apply_experts(self, x, ids, weights, w_gate_up, w_down, packed, shared, shared_gate):
         T, n = x.shape
+        E = w_gate_up.shape[0]
         ff = w_gate_up.shape[1] // 2
         xf = x.to(torch.float32)
         out = torch.zeros(T, n)
         for t in range(T):
             for j in range(ids.shape[1]):
                 e = int(ids[t, j])
+                if e >= E:                          # an expert that hands its input on
+                    out[t] += weights[t, j] * xf[t]
+                    continue
                 gu = w_gate_up[e].to(torch.float32) @ xf[t]
                 a = (gu[:ff] / (1 + torch.exp(-gu[:ff])) * gu[ff:]).to(x.dtype).to(torch.float32)
                 out[t] += weights[t, j] * (w_down[e].to(torch.float32) @ a)
         if shared is not None:
-            out = out + shared_gate[:, None] * shared.to(torch.float32)
+            out = out + (shared.to(torch.float32) if shared_gate is None else shared_gate[:, None] * shared.to(torch.float32))
         return out.to(x.dtype)
+
+    # ---- blocks that norm what a sublayer gives; attention with sizes of its own ----
+    def residual_rows(self, resid, dtype):
+        return resid if dtype == torch.float32 else resid.to(dtype)
+
+    def norm_add(self, resid, y, weight, eps, out_dtype):
+        yf = y.to(torch.float32)
+        resid += weight * yf * torch.rsqrt((yf * yf).mean(dim=-1, keepdim=True) + eps)
+        return resid if out_dtype == torch.float32 else resid.to(out_dtype)
+
+    def check_sized_attention(self, heads, kv_heads, key_dim, value_dim):
+        pass
+
+    @staticmethod
+    def _seen(p, window, keep_first):
+        """The positions a row at p sees, ascending."""
+        if not window:
+            return torch.arange(0, p + 1)
+        lo = max(0, p - window + 1)
+        return torch.cat([torch.arange(0, min(keep_first, lo)), torch.arange(lo, p + 1)])
+
+    def differential_attention(self, proj, step, cache, heads, kv_heads, dim, vdim, q_weight, k_weight, norm_eps, scale,
+                               lam, after, window, keep_first):
+        T = step.num_rows
+        x = proj.to(torch.float32)
+        nq, nk, nv = heads * 2 * dim, kv_heads * 2 * dim, kv_heads * vdim
+
+        def norm(t, w):
+            return w * t * torch.rsqrt((t * t).mean(dim=-1, keepdim=True) + norm_eps)
+        q = norm(x[:, :nq].reshape(T, heads * 2, dim), q_weight).to(proj.dtype).to(torch.float32)
+        k = norm(x[:, nq:nq + nk].reshape(T, kv_heads * 2, dim), k_weight)
+        v = x[:, nq + nk:nq + nk + nv].reshape(T, kv_heads, vdim)
+        gate = torch.sigmoid(x[:, nq + nk + nv:])
+        page, tables = cache.group.page_size, cache.group.tables
+        pos, seq = step.positions.long(), step.seq_of_row.long()
+        pages = tables[seq, pos // page].long()
+        assert (pages >= 0).all(), "a row writes to a page that is not held"
+        kc, vc = cache.record("k"), cache.record("v")
+        kc[pages, :, pos % page] = k.to(kc.dtype)
+        vc[pages, :, :, pos % page] = v.to(vc.dtype)
+        out = torch.zeros(T, heads, vdim)
+        mul = heads // kv_heads
+        for r in range(T):
+            idx = self._seen(int(pos[r]), window, keep_first)
+            pg = tables[int(seq[r]), idx // page].long()
+            assert (pg >= 0).all(), "a row reads a page that is not held"
+            kk = kc[pg, :, idx % page].to(torch.float32)            # [n, kv * 2, dim]
+            vv = vc[pg, :, :, idx % page].to(torch.float32)         # [n, kv, vdim]
+            for h in range(heads):
+                g = h // mul
+                a = [torch.softmax((kk[:, g * 2 + m] @ q[r, h * 2 + m]) * scale, dim=0) @ vv[:, g] for m in range(2)]
+                o = a[0] - lam * a[1]
+                out[r, h] = o * torch.rsqrt((o * o).mean() + norm_eps) * after * gate[r, h]
+        return out.reshape(T, heads * vdim).to(proj.dtype)
+
+    def latent_attention(self, proj, step, cache, heads, dim, rot, rank, vdim, norm_weight, norm_eps, rotary, scale,
+                         w_qk, w_v):
+        T = step.num_rows
+        x = proj.to(torch.float32)
+        cos, sin, rd = rotary
+        half = rd // 2
+        pos, seq = step.positions.long(), step.seq_of_row.long()
+
+        def turn(t, c, s):
+            a, b, rest = t[..., :half], t[..., half:rd], t[..., rd:]
+            return torch.cat([a * c - b * s, b * c + a * s, rest], dim=-1)
+        q = x[:, :heads * (dim + rot)].reshape(T, heads, dim + rot)
+        down = x[:, heads * (dim + rot):]
+        c = down[:, :rank]
+        c = norm_weight * c * torch.rsqrt((c * c).mean(dim=-1, keepdim=True) + norm_eps)
+        entry = torch.cat([c, turn(down[:, rank:], cos[pos], sin[pos])], dim=-1)
+        page, tables = cache.group.page_size, cache.group.tables
+        pages = tables[seq, pos // page].long()
+        assert (pages >= 0).all(), "a row writes to a page that is not held"
+        kc = cache.record("latent")
+        kc[pages, pos % page] = entry.to(kc.dtype)
+        q_lat = torch.einsum("thd,hnd->thn", q[..., :dim].to(proj.dtype).to(torch.float32), w_qk.to(torch.float32))
+        qk = torch.cat([q_lat, turn(q[..., dim:], cos[pos][:, None], sin[pos][:, None])], dim=-1).to(proj.dtype).to(torch.float32)
+        o = torch.zeros(T, heads, rank)
+        for r in range(T):
+            idx = torch.arange(0, int(pos[r]) + 1)
+            pg = tables[int(seq[r]), idx // page].long()
+            assert (pg >= 0).all(), "a row reads a page that is not held"
+            kk = kc[pg, idx % page].to(torch.float32)               # [n, rank + rot]
+            w = torch.softmax((qk[r] @ kk.t()) * scale, dim=-1)     # [heads, n]
+            o[r] = w @ kk[:, :rank]
+        o = o.to(proj.dtype).to(torch.float32)
+        return torch.einsum("thn,hen->the", o, w_v.to(torch.float32)).reshape(T, heads * vdim).to(proj.dtype)
 
     def add_rmsnorm(self, resid, delta, weight, eps, out_dtype, rows=None, num_rows=None, lazy=False):
         if rows is None:

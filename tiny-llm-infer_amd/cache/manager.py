@@ -82,6 +82,7 @@ class CacheNeed:
     records: Tuple[CacheRecord, ...]
     window: Optional[int] = None
     chunk: Optional[int] = None          # rows read only inside their own block of ``chunk`` positions (counted from 0)
+    keep_first: int = 0                  # with a window: the first so many positions of a sequence stay readable for ever
 
     def __post_init__(self):
         names = [r.name for r in self.records]
@@ -91,6 +92,8 @@ class CacheNeed:
             raise ValueError("a cache need has a window or a chunk, not both")
         if (self.window is not None and self.window <= 0) or (self.chunk is not None and self.chunk <= 0):
             raise ValueError("a window or a chunk must be positive")
+        if self.keep_first < 0 or (self.keep_first and self.window is None):
+            raise ValueError("first positions are kept beside a window only, and their number cannot be negative")
 
     @property
     def keeps_all(self) -> bool:
@@ -191,14 +194,15 @@ def page_hash(tokens: Sequence[int], prefix_hash: int) -> int:
     return h
 
 
-def window_group_pages(window: int, page_size: int, max_requests: int, max_step_tokens: int) -> int:
+def window_group_pages(window: int, page_size: int, max_requests: int, max_step_tokens: int, keep_first: int = 0) -> int:
     """The most pages that the live requests of a window group can hold together.  A request that
     has s tokens in the cache and runs c more holds the blocks from the first one a query at s
     reads to the one its last token is written to: at most (window - 1 + c) / page + 2, the
-    window and the portion each straddling a page's edge.  Over ``max_requests`` requests whose
+    window and the portion each straddling a page's edge; and the blocks of the first
+    ``keep_first`` positions, which it never gives back.  Over ``max_requests`` requests whose
     portions of one step add up to ``max_step_tokens``."""
     blocks = lambda n: (n + page_size - 1) // page_size
-    return max_requests * (blocks(window - 1) + 2) + blocks(max_step_tokens)
+    return max_requests * (blocks(window - 1) + 2 + blocks(keep_first)) + blocks(max_step_tokens)
 
 
 def group_needs(needs: Sequence[Optional["CacheNeed"]]) -> List["CacheNeed"]:
@@ -226,7 +230,7 @@ class CacheManager:
         distinct = group_needs(needs)
         if per_group is None:
             per_group = [num_pages if (n.keeps_all or max_step_tokens is None) else
-                         min(num_pages, window_group_pages(n.reach, page_size, max_requests, max_step_tokens))
+                         min(num_pages, window_group_pages(n.reach, page_size, max_requests, max_step_tokens, n.keep_first))
                          for n in distinct]
         if len(per_group) != len(distinct):
             raise ValueError(f"{len(per_group)} page counts for {len(distinct)} groups of cache layers")
@@ -370,6 +374,11 @@ class CacheManager:
         """Lowest block a query at ``first_query_pos`` (and any later one) can read."""
         return g.need.first_read(first_query_pos) // self.page_size
 
+    def _kept_blocks(self, g: GroupLayout) -> int:
+        """The leading blocks of a request that a window group never gives back: those of the first
+        positions that every later row still reads."""
+        return _blocks(g.need.keep_first, self.page_size)
+
     def pages_needed(self, key: Hashable, new_total: int) -> List[int]:
         """Per group, pages that must be taken so that the request can run the
         tokens at positions [num_tokens, new_total)."""
@@ -400,7 +409,7 @@ class CacheManager:
             if g.need.keeps_all:
                 out.append(whole)
             else:
-                out.append(min(whole, _blocks(g.need.reach - 1, self.page_size) + 2
+                out.append(min(whole, _blocks(g.need.reach - 1, self.page_size) + 2 + self._kept_blocks(g)
                                + _blocks(min(portion, total_tokens), self.page_size)))
         return out
 
@@ -470,7 +479,7 @@ class CacheManager:
                 continue
             table = rc.tables[gi]
             first = min(self._first_needed_block(g, new_total), len(table))
-            for b in range(first):
+            for b in range(self._kept_blocks(g), first):
                 if table[b] >= 0:
                     g.pool.release(table[b])
                     self.pages_returned_total += 1
@@ -507,6 +516,8 @@ class CacheManager:
                 first = self._first_needed_block(g, rc.num_tokens)
                 if any(page < 0 for page in rc.tables[gi][first:]):
                     raise PageError(f"group {gi}: the table of {rc.key!r} has a hole at or after block {first}")
+                if any(page < 0 for page in rc.tables[gi][:self._kept_blocks(g)]):
+                    raise PageError(f"group {gi}: {rc.key!r} has lost a block of its first positions, which it keeps")
             for page in range(g.pool.num_pages):
                 if g.pool.ref_count(page) != held.get(page, 0):
                     raise PageError(f"group {gi} page {page}: pool counts "

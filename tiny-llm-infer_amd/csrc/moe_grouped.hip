@@ -46,9 +46,8 @@ __global__ void __launch_bounds__(1024) moe_sort_kernel(const int* __restrict__ 
     for (int e = threadIdx.x; e < E; e += blockDim.x) count[e] = fill[e] = 0;
     __syncthreads();
     for (int p = threadIdx.x; p < P; p += blockDim.x) {
-        int e = ids[p];
-        if (e < 0 || e >= E) e = 0;                   // (the router gives no such id)
-        atomicAdd(&count[e], 1);
+        const int e = ids[p];
+        if (e >= 0 && e < E) atomicAdd(&count[e], 1);   // (any other id: an expert that hands its input on, no slot)
     }
     __syncthreads();
     for (int e = threadIdx.x; e < E; e += blockDim.x) {
@@ -65,8 +64,11 @@ __global__ void __launch_bounds__(1024) moe_sort_kernel(const int* __restrict__ 
     for (int s = threadIdx.x; s < tiles_max * RT; s += blockDim.x) order[s] = -1;
     __syncthreads();
     for (int p = threadIdx.x; p < P; p += blockDim.x) {
-        int e = ids[p];
-        if (e < 0 || e >= E) e = 0;
+        const int e = ids[p];
+        if (e < 0 || e >= E) {
+            pos[p] = -1;
+            continue;
+        }
         const int slot = start[e] + atomicAdd(&fill[e], 1);
         order[slot] = p;
         pos[p] = slot;
@@ -307,13 +309,17 @@ __global__ void __launch_bounds__(256) moe_down_grouped_kernel(const bf16_t* __r
 // y[row] = sum_j weight[row, j] part[pos[row, j]] (+ gate[row] * shared[row])
 __global__ void moe_combine_kernel(const float* __restrict__ part, const int* __restrict__ pos,
                                    const float* __restrict__ weights, const bf16_t* __restrict__ shared,
-                                   const float* __restrict__ shared_gate, bf16_t* __restrict__ out, int top, int D) {
+                                   const float* __restrict__ shared_gate, bf16_t* __restrict__ out, int top, int D,
+                                   const bf16_t* __restrict__ x) {
     const int t = blockIdx.x;
     for (int cidx = threadIdx.x; cidx < D; cidx += blockDim.x) {
         float y = 0.f;
-        for (int j = 0; j < top; ++j)
-            y = fmaf(weights[(size_t)t * top + j], part[(size_t)pos[(size_t)t * top + j] * D + cidx], y);
-        if (shared) y = fmaf(shared_gate[t], bf16_to_f32(shared[(size_t)t * D + cidx]), y);
+        for (int j = 0; j < top; ++j) {
+            const int slot = pos[(size_t)t * top + j];           // negative: the expert hands its input on
+            const float v = slot >= 0 ? part[(size_t)slot * D + cidx] : bf16_to_f32(x[(size_t)t * D + cidx]);
+            y = fmaf(weights[(size_t)t * top + j], v, y);
+        }
+        if (shared) y = fmaf(shared_gate ? shared_gate[t] : 1.0f, bf16_to_f32(shared[(size_t)t * D + cidx]), y);
         out[(size_t)t * D + cidx] = f32_to_bf16(y);
     }
 }
@@ -342,7 +348,6 @@ extern "C" int tli_moe_grouped_bf16(const void* x, const int* ids, const float* 
                         SORT_MAX_EXPERTS, D, ff);
     if (RT != 16 && RT != 32 && RT != 64 && RT != 128)
         return tli_fail("moe_grouped: tiles of 16, 32, 64 or 128 slots, not %d", RT);
-    if (shared && !shared_gate) return tli_fail("moe_grouped: a shared expert without its gate");
     const long long pairs = (long long)T * top;
     const long long tiles_max = pairs / RT + E;
     if (tiles_max > 65535 || pairs > (1 << 28)) return tli_fail("moe_grouped: too many pairs for one launch (%lld)", pairs);
@@ -361,6 +366,6 @@ extern "C" int tli_moe_grouped_bf16(const void* x, const int* ids, const float* 
     else { TLI_GROUPED(8, 1); }
 #undef TLI_GROUPED
     hipLaunchKernelGGL(moe_combine_kernel, dim3(T), dim3(256), 0, s, part, pos, weights, (const bf16_t*)shared, shared_gate,
-                       (bf16_t*)out, top, D);
+                       (bf16_t*)out, top, D, (const bf16_t*)x);
     return tli_check_launch("moe_grouped");
 }

@@ -34,7 +34,7 @@ def window_bytes(model, page_size: int, max_batch_tokens: int, max_num_seqs: int
     total = 0
     for need in model.cache_needs():
         if need is not None and not need.keeps_all:
-            pages = window_group_pages(need.reach, page_size, max_num_seqs, max_batch_tokens)
+            pages = window_group_pages(need.reach, page_size, max_num_seqs, max_batch_tokens, need.keep_first)
             total += pages * need_page_bytes(need, page_size, model.env.dtype)
     return total
 

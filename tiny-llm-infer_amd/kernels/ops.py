@@ -109,8 +109,16 @@ def load_library():
         "tli_delta_recurrence": [P, P, P, P, P, P, P, P, P, P, P, I, I, I, I, I, P],
         "tli_delta_state_floats": [I, I],
         "tli_gated_rmsnorm": [P, P, I, P, P, I, I, I, F, I, P],
-        "tli_moe_route": [P, ctypes.c_longlong, ctypes.c_longlong, P, P, P, I, I, I, I, I, F, I, P],
-        "tli_moe_experts": [P, P, P, P, P, P, P, P, P, I, I, I, I, I, P],
+        "tli_moe_route": [P, ctypes.c_longlong, ctypes.c_longlong, P, P, P, I, I, I, I, I, F, I, I, I, I, P, P],
+        "tli_moe_experts": [P, P, P, P, P, P, P, P, P, I, I, I, I, I, I, P],
+        "tli_norm_add": [P, P, P, P, I, I, F, I, P],
+        "tli_residual_rows": [P, P, ctypes.c_longlong, P],
+        "tli_attention_sized_plain": [P, P, P, P, P, P, P, I, I, I, I, I, I, I, I, I, F, I, I, I, I, P],
+        "tli_diff_prepare": [P, I, P, P, P, P, P, P, I, I, I, I, I, I, I, I, P, P, F, I, P],
+        "tli_diff_combine": [P, P, I, I, P, I, I, I, F, F, F, I, P],
+        "tli_latent_prepare": [P, I, P, P, P, P, P, I, I, I, I, I, I, I, I, I, P, F, P, P, I, P],
+        "tli_head_products_plain": [P, ctypes.c_longlong, ctypes.c_longlong, P, P, ctypes.c_longlong, ctypes.c_longlong,
+                                    I, I, I, I, I, P],
         "tli_moe_grouped_tile": [I, I],
         "tli_moe_grouped_bf16": [P, P, P, P, P, P, P, P, P, P, P, P, P, P, P, I, I, I, I, I, I, P],
         "tli_sample": [P, I, I, P, P, P, P, P, P],
@@ -1184,9 +1192,24 @@ class HipOps:
                 "down": torch.stack([self.tile_matrix(w_down[e]) for e in range(E)]),
                 "experts": E, "hidden": n, "inter": ff}
 
-    def route_experts(self, z, experts, top, groups, keep, scale, has_shared, transposed=False):
+    ROUTER_SCORES = ("sigmoid", "softmax")
+    ROUTER_GROUP_SCORES = ("top2", "max")
+
+    def check_router(self, score: str, group_score: str) -> None:
+        if score not in self.ROUTER_SCORES or group_score not in self.ROUTER_GROUP_SCORES:
+            raise KernelError(f"a router with '{score}' scores and groups scored by '{group_score}' is not known; known: "
+                              f"{', '.join(self.ROUTER_SCORES)}; {', '.join(self.ROUTER_GROUP_SCORES)}")
+
+    def route_experts(self, z, experts, top, groups, keep, scale, has_shared, transposed=False, score="sigmoid",
+                      group_score="top2", normalize=True, correction=None):
         """From router logits ``z`` (float32 [T, E (+ 1)]; [E (+ 1), T] with ``transposed``) to the chosen experts (int32 [T, top]), their
-        weights (float32 [T, top]) and, if the last column is a shared expert's gate, its sigmoid [T]."""
+        weights (float32 [T, top]) and, if the last column is a shared expert's gate, its sigmoid [T].  ``score``: the
+        scores are the logits' sigmoid or their softmax over the E; ``correction`` (float32 [E]) is added to them for the
+        choice only; ``group_score``: a group counts by its two largest choice scores or by its largest; ``normalize``:
+        the chosen scores are divided by their sum."""
+        self.check_router(score, group_score)
+        if correction is not None:
+            self._want(correction, "router correction", torch.float32, (experts,))
         T = z.shape[1] if transposed else z.shape[0]
         columns = experts + (1 if has_shared else 0)
         self._want(z, "router logits", torch.float32, (columns, T) if transposed else (T, columns))
@@ -1195,13 +1218,15 @@ class HipOps:
         weights = torch.empty((T, top), dtype=torch.float32, device=self.device)
         gate = torch.empty((T,), dtype=torch.float32, device=self.device) if has_shared else None
         self._call(self.lib.tli_moe_route, z.data_ptr(), z_row, z_col, ids.data_ptr(), weights.data_ptr(), _ptr(gate), T,
-                   experts, top, groups, keep, float(scale), 1 if has_shared else 0, self._stream())
+                   experts, top, groups, keep, float(scale), 1 if has_shared else 0, self.ROUTER_SCORES.index(score),
+                   self.ROUTER_GROUP_SCORES.index(group_score), 1 if normalize else 0, _ptr(correction), self._stream())
         return ids, weights, gate
 
     def apply_experts(self, x, ids, weights, w_gate_up, w_down, packed, shared, shared_gate):
-        """sum_j weights[t, j] * expert ids[t, j] (x[t])  (+ shared_gate[t] * shared[t]);  ``w_gate_up``
-        [E, 2 ff, n] (an expert's gate rows, then its up rows), ``w_down`` [E, n, ff]; with ``packed`` (what
-        ``pack_experts`` gave) the row-major matrices may be None."""
+        """sum_j weights[t, j] * expert ids[t, j] (x[t])  (+ shared_gate[t] * shared[t], or + shared[t] without a
+        gate);  ``w_gate_up`` [E, 2 ff, n] (an expert's gate rows, then its up rows), ``w_down`` [E, n, ff]; with
+        ``packed`` (what ``pack_experts`` gave) the row-major matrices may be None.  An id from E on is an expert
+        that hands its input on: its term is weights[t, j] * x[t]."""
         T, n = x.shape
         top = ids.shape[1]
         self._want(x, "expert input")
@@ -1209,7 +1234,8 @@ class HipOps:
         self._want(weights, "experts' weights", torch.float32, (T, top))
         if shared is not None:
             self._want(shared, "shared expert's output", x.dtype, (T, n))
-            self._want(shared_gate, "shared expert's gate", torch.float32, (T,))
+            if shared_gate is not None:
+                self._want(shared_gate, "shared expert's gate", torch.float32, (T,))
         out = torch.empty((T, n), dtype=x.dtype, device=self.device)
         if T == 0:
             return out
@@ -1236,8 +1262,8 @@ class HipOps:
                            packed["gate"].data_ptr(), packed["up"].data_ptr(), packed["down"].data_ptr(), order.data_ptr(),
                            pos.data_ptr(), tile_expert.data_ptr(), num_tiles.data_ptr(), hid.data_ptr(), part.data_ptr(),
                            None if shared is None else shared[t0:t1].data_ptr(),
-                           None if shared is None else shared_gate[t0:t1].data_ptr(), out[t0:t1].data_ptr(), t1 - t0, top,
-                           E, n, ff, RT, self._stream())
+                           None if (shared is None or shared_gate is None) else shared_gate[t0:t1].data_ptr(),
+                           out[t0:t1].data_ptr(), t1 - t0, top, E, n, ff, RT, self._stream())
             return out
         if w_gate_up is None or w_down is None:
             raise KernelError("the experts' row-major matrices were not kept and the tiled ones do not apply here")
@@ -1251,9 +1277,159 @@ class HipOps:
             self._call(self.lib.tli_moe_experts, x[t0:t1].data_ptr(), ids[t0:t1].data_ptr(), weights[t0:t1].data_ptr(),
                        w_gate_up.data_ptr(), w_down.data_ptr(), hid[t0 * top:].data_ptr(),
                        None if shared is None else shared[t0:t1].data_ptr(),
-                       None if shared is None else shared_gate[t0:t1].data_ptr(), out[t0:t1].data_ptr(), t1 - t0, top, n, ff,
-                       _dtype_code(x.dtype), self._stream())
+                       None if (shared is None or shared_gate is None) else shared_gate[t0:t1].data_ptr(),
+                       out[t0:t1].data_ptr(), t1 - t0, top, n, ff, E, _dtype_code(x.dtype), self._stream())
         return out
+
+    # ---- blocks that norm what a sublayer gives ------------------------------------------------------------
+    def residual_rows(self, resid: torch.Tensor, dtype: torch.dtype) -> torch.Tensor:
+        """The float32 residual's rows in the run's type (the residual itself in a float32 run)."""
+        self._want(resid, "residual", torch.float32)
+        if dtype == torch.float32:
+            return resid
+        if dtype != torch.bfloat16:
+            raise KernelError(f"kernels take float32 or bfloat16 tensors, not {dtype}")
+        out = torch.empty(resid.shape, dtype=dtype, device=self.device)
+        self._call(self.lib.tli_residual_rows, resid.data_ptr(), out.data_ptr(), resid.numel(), self._stream())
+        return out
+
+    def norm_add(self, resid, y, weight, eps, out_dtype):
+        """resid (float32 [T, n]) += weight * y / sqrt(mean(y^2) + eps) with ``y`` [T, n] in the run's type (or an
+        unfinished product); returns the new residual's rows in the run's type (the residual itself in a float32 run)."""
+        y = self.resolve(y)
+        total, n = resid.shape
+        self._want(resid, "residual", torch.float32)
+        self._want(weight, "norm weight", torch.float32, (n,))
+        self._want(y, "sublayer output", out_dtype, (total, n))
+        out = resid if out_dtype == torch.float32 else torch.empty((total, n), dtype=out_dtype, device=self.device)
+        self._call(self.lib.tli_norm_add, resid.data_ptr(), y.data_ptr(), weight.data_ptr(),
+                   None if out is resid else out.data_ptr(), total, n, float(eps), _dtype_code(out_dtype), self._stream())
+        return out
+
+    # ---- attention whose keys and values have sizes of their own -------------------------------------------
+    MAX_SIZED_DIM = 1024
+
+    def check_sized_attention(self, heads: int, kv_heads: int, key_dim: int, value_dim: int) -> None:
+        if not (1 <= key_dim <= self.MAX_SIZED_DIM and 1 <= value_dim <= self.MAX_SIZED_DIM):
+            raise KernelError(f"heads of {key_dim} and {value_dim} elements are not supported: 1 to {self.MAX_SIZED_DIM}")
+        if heads <= 0 or kv_heads <= 0 or heads % kv_heads:
+            raise KernelError(f"{heads} heads cannot be grouped over {kv_heads} kv heads")
+
+    def _check_tables(self, g, step):
+        self._want(g.tables, "block tables", torch.int32, (step.num_seqs, g.table_width))
+        if (step.max_seq_len + g.page_size - 1) // g.page_size > g.table_width:
+            raise KernelError("a block table is narrower than its sequence needs")
+
+    def sized_attention(self, q, step, g, kc, vc, heads, kv_heads, maps, key_dim, value_dim, scale, window, keep_first,
+                        out_dtype):
+        """Attention of ``q`` [T, heads * maps, key_dim] over the key cache ``kc`` [pages, kv_heads * maps, page, key_dim]
+        and the value cache ``vc`` [pages, kv_heads, value_dim, page] (None: a key's first value_dim elements are its
+        values); map m of head h reads key head (h // (heads / kv_heads)) * maps + m.  A row at p sees t <= p with
+        p - t < window or t < keep_first (window None: all).  Returns [T, heads * maps, value_dim] of ``out_dtype``."""
+        T = step.num_rows
+        self.check_sized_attention(heads, kv_heads, key_dim, value_dim)
+        self._want(q, "queries", None, (T, heads * maps, key_dim))
+        pages = kc.shape[0]
+        self._want(kc, "key cache", q.dtype, (pages, kv_heads * maps, g.page_size, key_dim))
+        if vc is not None:
+            self._want(vc, "value cache", q.dtype, (pages, kv_heads, value_dim, g.page_size))
+        elif value_dim > key_dim:
+            raise KernelError("values that are the start of their keys cannot be longer than the keys")
+        self._check_tables(g, step)
+        if out_dtype not in (q.dtype, torch.float32):
+            raise KernelError(f"attention over {q.dtype} gives {q.dtype} or float32, not {out_dtype}")
+        out = torch.empty((T, heads * maps, value_dim), dtype=out_dtype, device=self.device)
+        self._call(self.lib.tli_attention_sized_plain, q.data_ptr(), out.data_ptr(), kc.data_ptr(), _ptr(vc),
+                   step.positions.data_ptr(), step.seq_of_row.data_ptr(), g.tables.data_ptr(), g.table_width, g.page_size,
+                   pages, T, heads, kv_heads, maps, key_dim, value_dim, float(scale), int(window or 0),
+                   int(keep_first or 0) if window else 0, _dtype_code(q.dtype), 1 if out_dtype == torch.float32 else 0,
+                   self._stream())
+        return out
+
+    def differential_attention(self, proj, step, cache, heads, kv_heads, dim, vdim, q_weight, k_weight, norm_eps, scale,
+                               lam, after, window, keep_first):
+        """Attention with two softmax maps a head, from the raw projections ``proj`` [T, q (heads * 2 * dim) | k
+        (kv_heads * 2 * dim) | v (kv_heads * vdim) | one gate logit a head] to the heads' gated outputs [T, heads *
+        vdim]: q and k normed per head and map (RMS norm, weights ``q_weight``, ``k_weight`` float32 [dim]), k and v
+        into the cache (records "k" [kv_heads * 2, page, dim] and "v" [kv_heads, vdim, page]), a1 and a2 the maps'
+        outputs over the same values, o = a1 - lam * a2, o / sqrt(mean(o^2) + norm_eps) * after * sigmoid(gate)."""
+        T = step.num_rows
+        width = (heads + kv_heads) * 2 * dim + kv_heads * vdim + heads
+        self._want(proj, "projections", None, (T, width))
+        for w in (q_weight, k_weight):
+            self._want(w, "head norm weight", torch.float32, (dim,))
+        if cache is None or not cache.writes:
+            raise KernelError("this attention writes its keys and values into a cache layer of its own")
+        kc, vc, g = cache.record("k"), cache.record("v"), cache.group
+        pages = kc.shape[0]
+        self._want(kc, "key cache", proj.dtype, (pages, kv_heads * 2, g.page_size, dim))
+        self._want(vc, "value cache", proj.dtype, (pages, kv_heads, vdim, g.page_size))
+        self._check_tables(g, step)
+        q = torch.empty((T, heads * 2, dim), dtype=proj.dtype, device=self.device)
+        self._call(self.lib.tli_diff_prepare, proj.data_ptr(), width, q.data_ptr(), kc.data_ptr(), vc.data_ptr(),
+                   step.positions.data_ptr(), step.seq_of_row.data_ptr(), g.tables.data_ptr(), g.table_width, g.page_size,
+                   pages, T, heads, kv_heads, dim, vdim, q_weight.data_ptr(), k_weight.data_ptr(), float(norm_eps),
+                   _dtype_code(proj.dtype), self._stream())
+        maps = self.sized_attention(q, step, g, kc, vc, heads, kv_heads, 2, dim, vdim, scale, window, keep_first,
+                                    torch.float32)
+        out = torch.empty((T, heads * vdim), dtype=proj.dtype, device=self.device)
+        self._call(self.lib.tli_diff_combine, maps.data_ptr(), proj.data_ptr(), width, width - heads, out.data_ptr(), T,
+                   heads, vdim, float(lam), float(after), float(norm_eps), _dtype_code(proj.dtype), self._stream())
+        return out
+
+    def head_products(self, x, x_stride, w, out=None, out_stride=None, x_at=0, out_at=0):
+        """y[t, h, :] = w[h] x[t, h, :] for a matrix a head, ``w`` [heads, N, K].  ``x`` is [T, columns]: the input of
+        head h are the K columns from ``x_at + h * x_stride`` on; ``out`` likewise with ``out_stride`` and ``out_at``
+        (made as [T, heads * N] if not given).  Float32 sums, results in the type of x."""
+        T, ldx = x.shape
+        heads, N, K = w.shape
+        self._want(x, "heads' inputs")
+        self._want(w, "matrices of the heads", x.dtype)
+        if x_at < 0 or x_stride < K or x_at + (heads - 1) * x_stride + K > ldx:
+            raise KernelError("a head's input lies outside its row")
+        if out is None:
+            out, out_stride, out_at = torch.empty((T, heads * N), dtype=x.dtype, device=self.device), N, 0
+        self._want(out, "heads' outputs", x.dtype)
+        if out.dim() != 2 or out.shape[0] != T or out_at < 0 or out_stride < N or out_at + (heads - 1) * out_stride + N > out.shape[1]:
+            raise KernelError("a head's output lies outside its row")
+        es = x.element_size()
+        self._call(self.lib.tli_head_products_plain, x.data_ptr() + x_at * es, ldx, x_stride, w.data_ptr(),
+                   out.data_ptr() + out_at * es, out.shape[1], out_stride, T, heads, N, K, _dtype_code(x.dtype), self._stream())
+        return out
+
+    def latent_attention(self, proj, step, cache, heads, dim, rot, rank, vdim, norm_weight, norm_eps, rotary, scale,
+                         w_qk, w_v):
+        """Attention whose keys and values are made from one latent vector a position, from the raw projections
+        ``proj`` [T, q (heads * (dim + rot)) | latent (rank) | key part (rot)] to the heads' outputs [T, heads * vdim].
+        The cache (record "latent" [page, rank + rot]) keeps the normed latent vector and the turned key part; a
+        head's score is q_plain . (W_uk c) + q_turned . k_turned, computed as (W_uk^T q_plain) . c with ``w_qk``
+        [heads, rank, dim] = W_uk^T a head, so that all heads read the one cached vector; the weighted sum of the
+        latent vectors then goes through ``w_v`` [heads, vdim, rank] = W_uv a head."""
+        T = step.num_rows
+        width = heads * (dim + rot) + rank + rot
+        self._want(proj, "projections", None, (T, width))
+        self._want(norm_weight, "latent norm weight", torch.float32, (rank,))
+        if cache is None or not cache.writes:
+            raise KernelError("this attention writes its latent vectors into a cache layer of its own")
+        kc, g = cache.record("latent"), cache.group
+        pages = kc.shape[0]
+        key = rank + rot
+        self._want(kc, "latent cache", proj.dtype, (pages, g.page_size, key))
+        self._check_tables(g, step)
+        cos, sin, rd = self._rotary(rotary, step)
+        if rd > rot:
+            raise KernelError(f"{rd} turned elements do not fit a key part of {rot}")
+        q = torch.empty((T, heads, key), dtype=proj.dtype, device=self.device)
+        self._call(self.lib.tli_latent_prepare, proj.data_ptr(), width, q.data_ptr(), kc.data_ptr(), step.positions.data_ptr(),
+                   step.seq_of_row.data_ptr(), g.tables.data_ptr(), g.table_width, g.page_size, pages, T, heads, dim, rot,
+                   rank, rd, norm_weight.data_ptr(), float(norm_eps), cos.data_ptr(), sin.data_ptr(),
+                   _dtype_code(proj.dtype), self._stream())
+        self._want(w_qk, "matrices into the latent space", proj.dtype, (heads, rank, dim))
+        self._want(w_v, "matrices out of the latent space", proj.dtype, (heads, vdim, rank))
+        self.head_products(proj, dim + rot, w_qk, out=q.view(T, heads * key), out_stride=key)
+        o = self.sized_attention(q, step, g, kc.view(pages, 1, g.page_size, key), None, heads, 1, 1, key, rank, scale,
+                                 None, 0, proj.dtype)
+        return self.head_products(o.view(T, heads * rank), rank, w_v)
 
     def sample(self, logits: torch.Tensor, temperatures: Optional[torch.Tensor] = None,
                seeds: Optional[torch.Tensor] = None, top_p: Optional[torch.Tensor] = None) -> torch.Tensor:

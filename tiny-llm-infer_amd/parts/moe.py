@@ -1,12 +1,17 @@
 """Routed experts: a feed-forward of E small gated feed-forwards of which every row uses ``top``,
 beside an optional shared one that every row uses.
 
-    s = sigmoid(W_router h)                                   [E], float32
-    the experts form ``groups`` equal groups of neighbours; a group's score is the sum of its two
-        largest s; experts outside the ``keep`` best groups cannot be chosen
-    chosen = the ``top`` largest s among the rest;  weight_j = s_j / (sum of the chosen s + 1e-20) * scale
-    out = sum_j weight_j expert_j(h)  +  sigmoid(w_sg . h) * shared(h)
-    expert(h) = W_down (silu(W_gate h) * (W_up h))
+    s = sigmoid(W_router h)   or   softmax(W_router h)        [E + I], float32     (``score``)
+    c = s + correction   (a vector of the checkpoint, where the spec names one): what the choice looks at
+    the router's outputs form ``groups`` equal groups of neighbours; a group's score is the sum of its two
+        largest c, or its largest c (``group_score``: "top2", "max"); outputs outside the ``keep`` best
+        groups cannot be chosen
+    chosen = the ``top`` largest c among the rest;  weight_j = s_j / (sum of the chosen s + 1e-20) * scale,
+        or s_j * scale (``normalize`` false)
+    out = sum_j weight_j expert_j(h)  +  sigmoid(w_sg . h) * shared(h)   (or + shared(h), where the spec
+        names no gate for the shared expert)
+    expert(h) = W_down (silu(W_gate h) * (W_up h));  the last I (``identity``) router outputs stand for
+        experts without matrices whose output is h itself
 
 The router's product gives float32 (the row of the shared expert's gate rides along as one more
 row of that matrix); scores, choice and weights are float32.  A row's chosen experts are added
@@ -30,7 +35,12 @@ class RoutedExperts(FeedForward):
         super().__init__(spec)
         p = spec.params
         self.hidden = int(p["hidden_size"])
-        self.experts = int(p["experts"])
+        self.experts = int(p["experts"])                  # experts with matrices
+        self.identity = int(p.get("identity") or 0)       # router outputs behind them whose expert hands h on
+        self.outputs = self.experts + self.identity
+        self.score = str(p.get("score", "sigmoid"))
+        self.group_score = str(p.get("group_score", "top2"))
+        self.normalize = bool(p.get("normalize", True))
         self.top = int(p["top"])
         self.groups = int(p.get("groups") or 1)
         self.keep = int(p.get("keep") or self.groups)
@@ -38,16 +48,20 @@ class RoutedExperts(FeedForward):
         self.inter = int(p["intermediate_size"])
         shared = p.get("shared_intermediate_size")
         self.shared_inter = None if shared is None else int(shared)
-        if self.experts % self.groups or not 1 <= self.keep <= self.groups \
-                or not 1 <= self.top <= self.keep * (self.experts // self.groups):
-            raise ValueError(f"{self.experts} experts in {self.groups} groups, {self.keep} kept, cannot give {self.top}")
+        if self.experts < 1 or self.outputs % self.groups or not 1 <= self.keep <= self.groups \
+                or not 1 <= self.top <= self.keep * (self.outputs // self.groups):
+            raise ValueError(f"{self.outputs} router outputs in {self.groups} groups, {self.keep} kept, cannot give {self.top}")
+        self.correction_name = spec.names.get("correction")
+        self.shared_gated = "shared_scale" in spec.names
 
     def _expert(self, j: int, role: str) -> str:
         return self.spec.names["experts"].format(j) + role
 
     def tensors(self) -> List[TensorDecl]:
         n = self.spec.names
-        out = [TensorDecl(n["router"], (self.experts, self.hidden))]
+        out = [TensorDecl(n["router"], (self.outputs, self.hidden))]
+        if self.correction_name is not None:
+            out.append(TensorDecl(self.correction_name, (self.outputs,)))
         for j in range(self.experts):
             out += [TensorDecl(self._expert(j, "gate"), (self.inter, self.hidden)),
                     TensorDecl(self._expert(j, "up"), (self.inter, self.hidden)),
@@ -55,15 +69,22 @@ class RoutedExperts(FeedForward):
         if self.shared_inter is not None:
             out += [TensorDecl(n["shared_gate"], (self.shared_inter, self.hidden)),
                     TensorDecl(n["shared_up"], (self.shared_inter, self.hidden)),
-                    TensorDecl(n["shared_down"], (self.hidden, self.shared_inter)),
-                    TensorDecl(n["shared_scale"], (1, self.hidden))]
+                    TensorDecl(n["shared_down"], (self.hidden, self.shared_inter))]
+            if self.shared_gated:
+                out.append(TensorDecl(n["shared_scale"], (1, self.hidden)))
         return out
 
     def load(self, weights: Dict[str, torch.Tensor], env: BuildEnv) -> None:
         super().load(weights, env)
         n = self.spec.names
-        env.ops.check_expert_sizes(self.experts, self.top, self.groups, self.keep, self.hidden, self.inter)
-        rows = [weights[n["router"]]] + ([weights[n["shared_scale"]]] if self.shared_inter is not None else [])
+        env.ops.check_expert_sizes(self.outputs, self.top, self.groups, self.keep, self.hidden, self.inter)
+        if (self.score, self.group_score) != ("sigmoid", "top2"):
+            env.ops.check_router(self.score, self.group_score)
+        self.has_gate = self.shared_inter is not None and self.shared_gated
+        rows = [weights[n["router"]]] + ([weights[n["shared_scale"]]] if self.has_gate else [])
+        self.correction = None
+        if self.correction_name is not None:
+            self.correction = weights[self.correction_name].to(torch.float32).contiguous()
         self.w_router = torch.cat([r.to(env.dtype) for r in rows], dim=0).contiguous()       # few rows: kept row-major
         # the experts' matrices side by side: [E, 2 ff, hidden] (an expert's gate rows, then its up rows), [E, hidden, ff]
         self.w_gate_up = torch.stack([torch.cat([weights[self._expert(j, "gate")], weights[self._expert(j, "up")]], dim=0)
@@ -80,13 +101,16 @@ class RoutedExperts(FeedForward):
             self.shared_down = as_matrix(weights[n["shared_down"]], env)
 
     def workspace_elems(self, rows: int) -> int:
-        return rows * (self.top * (3 * self.inter + self.hidden) + 3 * (self.shared_inter or 0) + 2 * self.experts)
+        return rows * (self.top * (3 * self.inter + self.hidden) + 3 * (self.shared_inter or 0) + 2 * self.outputs)
 
     def forward(self, x: torch.Tensor, step: StepView):
         ops = self.env.ops
         z, transposed = ops.small_product(x, self.w_router)
-        ids, weights, shared_gate = ops.route_experts(z, self.experts, self.top, self.groups, self.keep, self.scale,
-                                                      self.shared_inter is not None, transposed)
+        how = {}
+        if (self.score, self.group_score, self.normalize, self.correction) != ("sigmoid", "top2", True, None):
+            how = dict(score=self.score, group_score=self.group_score, normalize=self.normalize, correction=self.correction)
+        ids, weights, shared_gate = ops.route_experts(z, self.outputs, self.top, self.groups, self.keep, self.scale,
+                                                      self.has_gate, transposed, **how)
         shared = None
         if self.shared_inter is not None:
             shared = ops.linear(ops.linear_swiglu(x, self.shared_gate_up), self.shared_down)
