@@ -122,3 +122,72 @@ extern "C" int tli_head_products_plain(const void* x, long long x_row, long long
         return tli_fail("head_products: unknown dtype %d", dtype);
     return tli_check_launch("head_products_plain");
 }
+
+// ---------------------------------------------------------------------------------------------------------------
+// head_products on the matrix cores (bfloat16, N and K in sixteens): a workgroup of four waves takes 16 rows and one
+// head; its waves share out the head's blocks of 16 outputs.  A is a block of W (16 outputs x 16 of k), B the rows'
+// fragments, which a wave holds in registers for all its blocks (k up to 640), so a lane ends with four consecutive
+// outputs of one row.  v_mfma_f32_16x16x16_bf16.
+// ---------------------------------------------------------------------------------------------------------------
+typedef __attribute__((ext_vector_type(4))) short hp_bf16x4;
+typedef __attribute__((ext_vector_type(4))) float hp_f32x4;
+union HpFrag {
+    uint2 u;
+    hp_bf16x4 v;
+};
+
+template <int KM>
+__global__ __launch_bounds__(256) void head_products_mfma_kernel(const bf16_t* __restrict__ x, long long x_row, long long x_head,
+                                                                 const bf16_t* __restrict__ w, bf16_t* __restrict__ y,
+                                                                 long long y_row, long long y_head, int T, int N, int K) {
+    const int lane = threadIdx.x % 64, wave = threadIdx.x / 64;
+    const int col = lane % 16, grp = lane / 16;
+    const int t0 = blockIdx.x * 16, h = blockIdx.y;
+    const int t = min(t0 + col, T - 1);                                 // (rows past the end repeat the last; never stored)
+    const int nk = K / 16;
+    HpFrag xf[KM];
+    const bf16_t* xr = x + (size_t)t * x_row + (size_t)h * x_head;
+#pragma unroll
+    for (int j = 0; j < KM; ++j)
+        if (j < nk) xf[j].u = *reinterpret_cast<const uint2*>(xr + j * 16 + grp * 4);
+    for (int nb = wave; nb * 16 < N; nb += 4) {
+        const bf16_t* wr = w + ((size_t)h * N + nb * 16 + col) * K + grp * 4;
+        hp_f32x4 acc = (hp_f32x4){0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+        for (int j = 0; j < KM; ++j) {
+            if (j < nk) {
+                HpFrag a;
+                a.u = *reinterpret_cast<const uint2*>(wr + j * 16);
+                acc = __builtin_amdgcn_mfma_f32_16x16x16bf16_1k(a.v, xf[j].v, acc, 0, 0, 0);
+            }
+        }
+        if (t0 + col < T) {
+            uint2 st;
+            st.x = pack_bf16x2(acc[0], acc[1]);
+            st.y = pack_bf16x2(acc[2], acc[3]);
+            *reinterpret_cast<uint2*>(y + (size_t)t * y_row + (size_t)h * y_head + nb * 16 + grp * 4) = st;
+        }
+    }
+}
+
+extern "C" int tli_head_products_mfma_takes(int N, int K, long long x_row, long long x_head, long long y_row, long long y_head) {
+    return (N % 16 == 0 && K % 16 == 0 && N >= 16 && K >= 16 && K <= 640 && x_row % 4 == 0 && x_head % 4 == 0 &&
+            y_row % 4 == 0 && y_head % 4 == 0) ? 1 : 0;
+}
+
+extern "C" int tli_head_products_mfma_bf16(const void* x, long long x_row, long long x_head, const void* w, void* y,
+                                           long long y_row, long long y_head, int rows, int heads, int N, int K, void* stream) {
+    if (rows <= 0) return 0;
+    if (heads <= 0 || heads > 65535 || !tli_head_products_mfma_takes(N, K, x_row, x_head, y_row, y_head))
+        return tli_fail("head_products: the matrix-core kernel takes sizes in sixteens (k up to 640), not %d x %d", N, K);
+    if ((((uintptr_t)x | (uintptr_t)w | (uintptr_t)y) & 7)) return tli_fail("head_products: operands must be 8-byte aligned");
+    const dim3 grid((rows + 15) / 16, heads);
+    hipStream_t s = (hipStream_t)stream;
+    if (K <= 128)
+        head_products_mfma_kernel<8><<<grid, 256, 0, s>>>((const bf16_t*)x, x_row, x_head, (const bf16_t*)w, (bf16_t*)y, y_row, y_head,
+                                                         rows, N, K);
+    else
+        head_products_mfma_kernel<40><<<grid, 256, 0, s>>>((const bf16_t*)x, x_row, x_head, (const bf16_t*)w, (bf16_t*)y, y_row, y_head,
+                                                          rows, N, K);
+    return tli_check_launch("head_products_mfma");
+}

@@ -114,6 +114,11 @@ def load_library():
         "tli_norm_add": [P, P, P, P, I, I, F, I, P],
         "tli_residual_rows": [P, P, ctypes.c_longlong, P],
         "tli_attention_sized_plain": [P, P, P, P, P, P, P, I, I, I, I, I, I, I, I, I, F, I, I, I, I, P],
+        "tli_attention_sized_mfma_takes": [I, I, I, I],
+        "tli_head_products_mfma_takes": [I, I] + [ctypes.c_longlong] * 4,
+        "tli_head_products_mfma_bf16": [P, ctypes.c_longlong, ctypes.c_longlong, P, P, ctypes.c_longlong, ctypes.c_longlong,
+                                        I, I, I, I, P],
+        "tli_attention_sized_mfma_bf16": [P, P, P, P, P, P, I, I, P, I, I, I, I, I, I, I, I, F, I, I, I, I, P],
         "tli_diff_prepare": [P, I, P, P, P, P, P, P, I, I, I, I, I, I, I, I, P, P, F, I, P],
         "tli_diff_combine": [P, P, I, I, P, I, I, I, F, F, F, I, P],
         "tli_latent_prepare": [P, I, P, P, P, P, P, I, I, I, I, I, I, I, I, I, P, F, P, P, I, P],
@@ -1339,10 +1344,22 @@ class HipOps:
         if out_dtype not in (q.dtype, torch.float32):
             raise KernelError(f"attention over {q.dtype} gives {q.dtype} or float32, not {out_dtype}")
         out = torch.empty((T, heads * maps, value_dim), dtype=out_dtype, device=self.device)
+        keep = int(keep_first or 0) if window else 0
+        if (q.dtype == torch.bfloat16 and not self.force_plain
+                and self.lib.tli_attention_sized_mfma_takes(key_dim, value_dim, g.page_size, 0 if vc is None else 1)):
+            # tiles of 16 rows of a sequence; in steps of single rows a tile is a row, its columns the heads of a key head
+            grouped = 1 if step.max_rows_per_seq == 1 else 0
+            starts = step.h_row_start
+            tiles = T if grouped else sum((starts[i + 1] - starts[i] + 15) // 16 for i in range(step.num_seqs))
+            self._call(self.lib.tli_attention_sized_mfma_bf16, q.data_ptr(), out.data_ptr(), kc.data_ptr(), _ptr(vc),
+                       step.row_start.data_ptr(), step.seq_start.data_ptr(), step.num_seqs, tiles, g.tables.data_ptr(),
+                       g.table_width, g.page_size, pages, heads, kv_heads, maps, key_dim, value_dim, float(scale),
+                       int(window or 0), keep, grouped, 1 if out_dtype == torch.float32 else 0, self._stream())
+            return out
         self._call(self.lib.tli_attention_sized_plain, q.data_ptr(), out.data_ptr(), kc.data_ptr(), _ptr(vc),
                    step.positions.data_ptr(), step.seq_of_row.data_ptr(), g.tables.data_ptr(), g.table_width, g.page_size,
                    pages, T, heads, kv_heads, maps, key_dim, value_dim, float(scale), int(window or 0),
-                   int(keep_first or 0) if window else 0, _dtype_code(q.dtype), 1 if out_dtype == torch.float32 else 0,
+                   keep, _dtype_code(q.dtype), 1 if out_dtype == torch.float32 else 0,
                    self._stream())
         return out
 
@@ -1393,6 +1410,11 @@ class HipOps:
         if out.dim() != 2 or out.shape[0] != T or out_at < 0 or out_stride < N or out_at + (heads - 1) * out_stride + N > out.shape[1]:
             raise KernelError("a head's output lies outside its row")
         es = x.element_size()
+        if (x.dtype == torch.bfloat16 and not self.plain_products and x_at % 4 == 0 and out_at % 4 == 0
+                and self.lib.tli_head_products_mfma_takes(N, K, ldx, x_stride, out.shape[1], out_stride)):
+            self._call(self.lib.tli_head_products_mfma_bf16, x.data_ptr() + x_at * es, ldx, x_stride, w.data_ptr(),
+                       out.data_ptr() + out_at * es, out.shape[1], out_stride, T, heads, N, K, self._stream())
+            return out
         self._call(self.lib.tli_head_products_plain, x.data_ptr() + x_at * es, ldx, x_stride, w.data_ptr(),
                    out.data_ptr() + out_at * es, out.shape[1], out_stride, T, heads, N, K, _dtype_code(x.dtype), self._stream())
         return out
