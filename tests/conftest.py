@@ -44,3 +44,19 @@ def kapanex_clear_folders(tmp_path_factory):
     from kapanex_helpers import SMALL, make_folder
     root = tmp_path_factory.mktemp("kapanex_clear")
     return {name: make_folder(str(root / name), name, clear_routing=True) for name in SMALL}
+
+
+@pytest.fixture(scope="session")
+def gimipel_folders(tmp_path_factory):
+    """Model folders of the small Gimipel configurations, made once in a temporary folder."""
+    from gimipel_helpers import SMALL, make_folder
+    root = tmp_path_factory.mktemp("gimipel")
+    return {name: make_folder(str(root / name), name) for name in SMALL}
+
+
+@pytest.fixture(scope="session")
+def gimipel_clear_folders(tmp_path_factory):
+    """The same configurations with weights whose routers read nothing that rounding touches (for comparisons in bfloat16)."""
+    from gimipel_helpers import SMALL, make_folder
+    root = tmp_path_factory.mktemp("gimipel_clear")
+    return {name: make_folder(str(root / name), name, clear_routing=True) for name in SMALL}

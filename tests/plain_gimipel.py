@@ -9,12 +9,37 @@ n1, n2 RMS norms of the sublayer's output; the sublayers read x itself.
 """
 from __future__ import annotations
 
+import json
 import math
+import os
+import struct
 from typing import Dict, List, Optional
 
 import torch
 
 F = torch.float64
+
+
+def read_safetensors(path: str) -> Dict[str, torch.Tensor]:
+    kinds = {"BF16": torch.bfloat16, "F16": torch.float16, "F32": torch.float32, "I32": torch.int32}
+    with open(path, "rb") as fh:
+        raw = fh.read()
+    (hlen,) = struct.unpack("<Q", raw[:8])
+    header = json.loads(raw[8:8 + hlen])
+    out = {}
+    for name, info in header.items():
+        if name == "__metadata__":
+            continue
+        b, e = info["data_offsets"]
+        t = torch.frombuffer(bytearray(raw[8 + hlen + b:8 + hlen + e]), dtype=kinds[info["dtype"]]).reshape(info["shape"])
+        out[name] = t.to(F) if t.dtype.is_floating_point else t.clone()
+    return out
+
+
+def read_model(folder: str):
+    with open(os.path.join(folder, "config.json")) as fh:
+        cfg = json.load(fh)
+    return cfg, read_safetensors(os.path.join(folder, "model.safetensors"))
 
 
 def rms_norm(x: torch.Tensor, weight: Optional[torch.Tensor], eps: float) -> torch.Tensor:
