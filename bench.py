@@ -66,14 +66,14 @@ DESIGN_SIZES = {
 
 
 def compare_designs(args):
-    """Prefill and decode of the Sinepel design (or, with --design-names, of others: Kapanex) beside the Qwen3
+    """Prefill and decode of the Sinepel design (or, with --design-names, of others: Kapanex, Gimipel) beside the Qwen3
     dense decoder at equal layer sizes
     (random bfloat16 weights, 4 layers unless --layers says otherwise), through the step function:
     one prompt of --prefill-tokens in one step, and decode steps of --batch and 64 requests at
     --prompt-len tokens of context.  One JSON line."""
     import torch
 
-    from tiny_llm_infer_amd.config import KapanexConfig, Qwen3Config, SinepelConfig
+    from tiny_llm_infer_amd.config import GimipelConfig, KapanexConfig, Qwen3Config, SinepelConfig
     from tiny_llm_infer_amd.engine.loading import random_model
     from tiny_llm_infer_amd.engine.runner import ModelRunner, StepEntry
     import random
@@ -113,7 +113,24 @@ def compare_designs(args):
                        {"type": "delta", "mlp": moe,
                         "mixer": {"heads": heads, "kv_heads": kv_heads, "dim": dim, "vdim": dim, "conv": 4}}
                        for i in range(layers)]})
-        known = {"sinepel": ("Sinepel", sinepel), "kapanex": ("Kapanex", kapanex), "qwen3": ("Qwen3ForCausalLM", qwen)}
+        # Gimipel: attention with two maps a head (each of half the head size, so a head's scores cost what Qwen3's
+        # do; a window of 1,024 beside the first 4 keys) and latent attention (a latent vector of 4 heads' size and a
+        # turned part of half a head for all heads) in turn; 15 experts and one that hands its input on, otherwise
+        # the feed-forward of Kapanex above
+        gmoe = {"kind": "moe", "expert": {"ff": ff // 4}, "shared": {"ff": ff // 2},
+                "router": {"experts": 15, "identity": 1, "top": 2, "groups": {"count": 4, "keep": 2}}}
+        gimipel = GimipelConfig.from_dict({
+            "architecture": "Gimipel", "vocab": vocab, "width": width, "embedding": {"scale": 1.0}, "norm": {"eps": 1e-5},
+            "max_positions": context,
+            "layers": [{"type": "attention", "mlp": gmoe,
+                        "mixer": {"heads": heads, "kv_heads": kv_heads, "dim": dim // 2, "vdim": dim, "scale": (dim // 2) ** -0.5,
+                                  "diff": 0.5, "mask": {"size": 1024, "keep_first": 4}}} if i % 2 == 0 else
+                       {"type": "latent_attention", "mlp": gmoe,
+                        "mixer": {"heads": heads, "dim": dim, "rot_dim": dim // 2, "vdim": dim, "kv_rank": 4 * dim,
+                                  "scale": (dim + dim // 2) ** -0.5, "rot": {"dims": dim // 2, "base": 1e6}}}
+                       for i in range(layers)]})
+        known = {"sinepel": ("Sinepel", sinepel), "kapanex": ("Kapanex", kapanex), "gimipel": ("Gimipel", gimipel),
+                 "qwen3": ("Qwen3ForCausalLM", qwen)}
         names = [n for n in args.design_names.split(",") if n]
         if any(n not in known for n in names):
             print(f"--design-names: known designs are {', '.join(known)}")
@@ -194,7 +211,7 @@ def main():
                     help="instead of the default workload: the Sinepel design beside the Qwen3 dense decoder at equal layer "
                          f"sizes, prefill and decode; a list of {','.join(DESIGN_SIZES)} or 'all'")
     ap.add_argument("--design-names", default="sinepel,qwen3",
-                    help="with --designs: which designs are run at every size (sinepel, kapanex, qwen3)")
+                    help="with --designs: which designs are run at every size (sinepel, kapanex, gimipel, qwen3)")
     args = ap.parse_args()
     if args.gpus != 1:
         print(f"bench.py runs on one GPU only; --gpus {args.gpus} is not supported (single-GPU engine)")

@@ -71,8 +71,10 @@ SMALL = {
 }
 
 
-def make_weights(cfg: dict, seed: int, clear_routing: bool = False) -> Dict[str, torch.Tensor]:
-    """bfloat16 weights of a size that makes every mechanism show in the logits.  ``clear_routing``: no router's
+def make_weights(cfg: dict, seed: int, clear_routing: bool = False, mild: bool = False) -> Dict[str, torch.Tensor]:
+    """bfloat16 weights of a size that makes every mechanism show in the logits.  ``mild``: scores a quarter as
+    large, so that a softmax does not multiply the rounding of bfloat16 queries and keys (scores of 20 and more move
+    by a tenth when their inputs are rounded, and so do the weights made of them).  ``clear_routing``: no router's
     logits depend on anything that rounding touches, so that a run in bfloat16 chooses as the plain implementation
     does (a row that goes to another expert is another computation, and so are the rows behind it).  The last n
     elements of the width are set aside (n router outputs): a token's embedding has one of them set (which one: its
@@ -80,6 +82,7 @@ def make_weights(cfg: dict, seed: int, clear_routing: bool = False) -> Dict[str,
     weight 3 / n (((p(e) + j) mod n) - (n - 1) / 2) for a permutation p a layer; all of it exact in bfloat16."""
     g = torch.Generator().manual_seed(seed)
     D = cfg["width"]
+    sharp = 0.5 if mild else 1.0
 
     def normal(*shape, std=1.0, mean=0.0):
         return torch.randn(*shape, generator=g) * std + mean
@@ -98,13 +101,13 @@ def make_weights(cfg: dict, seed: int, clear_routing: bool = False) -> Dict[str,
             w[p + "mix.v"] = normal(G * e, D, std=D ** -0.5 * 1.5)
             w[p + "mix.g"] = normal(H, D, std=D ** -0.5 * 2)
             w[p + "mix.o"] = normal(D, H * e, std=(H * e) ** -0.5 * 1.5)
-            w[p + "mix.q.norm"] = normal(d, std=0.2, mean=2.0)
-            w[p + "mix.k.norm"] = normal(d, std=0.2, mean=2.0)
+            w[p + "mix.q.norm"] = normal(d, std=0.2 * sharp, mean=2.0 * sharp)
+            w[p + "mix.k.norm"] = normal(d, std=0.2 * sharp, mean=2.0 * sharp)
             for r in ("lq1", "lk1", "lq2", "lk2"):
                 w[p + "mix." + r] = normal(d, std=0.15)
         else:
             H, d, r, e, n = m["heads"], m["dim"], m["rot_dim"], m["vdim"], m["kv_rank"]
-            w[p + "mix.q"] = normal(H * (d + r), D, std=D ** -0.5 * 3)
+            w[p + "mix.q"] = normal(H * (d + r), D, std=D ** -0.5 * 3 * sharp * sharp)
             w[p + "mix.dkv"] = normal(n + r, D, std=D ** -0.5 * 2)
             w[p + "mix.dkv.norm"] = normal(n, std=0.1, mean=1.0)
             w[p + "mix.uk"] = normal(H * d, n, std=n ** -0.5 * 2)
@@ -152,15 +155,29 @@ def write_folder(folder: str, cfg: dict, weights: Dict[str, torch.Tensor]) -> st
     return folder
 
 
-def make_folder(folder: str, name: str, clear_routing: bool = False) -> str:
+def make_folder(folder: str, name: str, clear_routing: bool = False, mild: bool = False) -> str:
     cfg, _, seed = SMALL[name]
-    return write_folder(folder, cfg, make_weights(cfg, seed, clear_routing=clear_routing))
+    return write_folder(folder, cfg, make_weights(cfg, seed, clear_routing=clear_routing, mild=mild))
 
 
 def plain_logits(folder: str, reqs: Dict[str, List[int]]) -> Dict[str, np.ndarray]:
     import plain_gimipel
     cfg, w = plain_gimipel.read_model(folder)
     return {rid: plain_gimipel.forward(cfg, w, toks).numpy() for rid, toks in reqs.items()}
+
+
+def rows_with_a_clear_choice(folder: str, reqs: Dict[str, List[int]], margin: float) -> Dict[str, int]:
+    """For every request, the number of leading rows whose routers all choose by more than ``margin``.  Rounding
+    in bfloat16 can turn a closer call, after which that row and the rows behind it are another computation."""
+    import plain_gimipel
+    cfg, w = plain_gimipel.read_model(folder)
+    out = {}
+    for rid, toks in reqs.items():
+        margins = []
+        plain_gimipel.forward(cfg, w, toks, margins=margins)
+        close = [any(layer[t] < margin for layer in margins) for t in range(len(toks))]
+        out[rid] = close.index(True) if True in close else len(toks)
+    return out
 
 
 def plain_greedy(folder: str, prompt: List[int], new_tokens: int) -> List[int]:

@@ -127,8 +127,10 @@ def gated_ff(h: torch.Tensor, w: Dict[str, torch.Tensor], p: str) -> torch.Tenso
     return ((z * torch.sigmoid(z)) * (h @ w[p + "up"].T)) @ w[p + "down"].T
 
 
-def route(h: torch.Tensor, f: Dict, w: Dict[str, torch.Tensor], p: str):
-    """Per position the chosen router outputs and their weights (lists of lists)."""
+def route(h: torch.Tensor, f: Dict, w: Dict[str, torch.Tensor], p: str, margins: Optional[list] = None):
+    """Per position the chosen router outputs and their weights (lists of lists).  ``margins``: a list
+    that takes, per position, by how much the choice was made (the smallest difference of choice scores
+    between a group or an output that was taken and one that was not)."""
     r = f["router"]
     E, ident, top = r["experts"], int(r.get("identity", 0)), r["top"]
     groups = r.get("groups") or {}
@@ -141,20 +143,27 @@ def route(h: torch.Tensor, f: Dict, w: Dict[str, torch.Tensor], p: str):
     ids, weights = [], []
     for t in range(h.shape[0]):
         c = choice[t].clone()
+        margin = float("inf")
         if keep < count:
             best = c.view(count, per).max(dim=1).values
             order = sorted(range(count), key=lambda g: (-float(best[g]), g))
+            margin = float(best[order[keep - 1]] - best[order[keep]])
             for g in order[keep:]:
                 c[g * per:(g + 1) * per] = float("-inf")
-        chosen = sorted(range(n), key=lambda j: (-float(c[j]), j))[:top]
+        ranked = sorted(range(n), key=lambda j: (-float(c[j]), j))
+        chosen = ranked[:top]
+        if top < n and c[ranked[top]] > float("-inf"):
+            margin = min(margin, float(c[ranked[top - 1]] - c[ranked[top]]))
+        if margins is not None:
+            margins.append(margin)
         ids.append(chosen)
         weights.append([float(s[t, j]) for j in chosen])
     return ids, weights
 
 
-def routed_experts(h: torch.Tensor, f: Dict, w: Dict[str, torch.Tensor], p: str) -> torch.Tensor:
+def routed_experts(h: torch.Tensor, f: Dict, w: Dict[str, torch.Tensor], p: str, margins: Optional[list] = None) -> torch.Tensor:
     E = f["router"]["experts"]
-    ids, weights = route(h, f, w, p)
+    ids, weights = route(h, f, w, p, margins)
     out = torch.zeros_like(h)
     for t in range(h.shape[0]):
         row = h[t:t + 1]
@@ -171,9 +180,11 @@ def owner(cfg: Dict, i: int) -> int:
     return i
 
 
-def forward(cfg: Dict, w: Dict[str, torch.Tensor], tokens: List[int], residuals: Optional[list] = None) -> torch.Tensor:
+def forward(cfg: Dict, w: Dict[str, torch.Tensor], tokens: List[int], residuals: Optional[list] = None,
+            margins: Optional[list] = None) -> torch.Tensor:
     """Logits [T, vocab] of one whole sequence.  ``residuals``: a list that takes the residual
-    stream after every layer."""
+    stream after every layer; ``margins``: one that takes, layer by layer, a list of every position's
+    margin of the router's choice."""
     eps = float(cfg["norm"]["eps"])
     x = w["embed"][torch.tensor(tokens)] * float((cfg.get("embedding") or {}).get("scale", 1.0))
     for i, layer in enumerate(cfg["layers"]):
@@ -186,7 +197,10 @@ def forward(cfg: Dict, w: Dict[str, torch.Tensor], tokens: List[int], residuals:
             raise ValueError(layer["type"])
         x = x + rms_norm(a, w[p + "norm1"], eps)
         if layer.get("mlp") is not None:
-            x = x + rms_norm(routed_experts(x, layer["mlp"], w, p + "mlp."), w[p + "norm2"], eps)
+            by_row = None if margins is None else []
+            x = x + rms_norm(routed_experts(x, layer["mlp"], w, p + "mlp.", by_row), w[p + "norm2"], eps)
+            if margins is not None:
+                margins.append(by_row)
         if residuals is not None:
             residuals.append(x.clone())
     return rms_norm(x, w["final.norm"], eps) @ w["head"].T

@@ -1,0 +1,411 @@
+"""Gimipel on the GPU: each mechanism's kernels alone against the plain implementation's function
+for it, then the model through the step function in every cut, in float32 and in bfloat16, keys at
+the window's edge and at the edge of the kept first ones, a key hundreds of positions back, long
+decoding through recorded launches, and greedy generation through the engine and the command line."""
+import json
+import os
+import subprocess
+import sys
+
+import numpy as np
+import pytest
+import torch
+
+import plain_gimipel
+from gimipel_helpers import (SMALL, _attention, _config, _latent, _layer, _moe, make_weights, plain_greedy, plain_logits,
+                             rows_with_a_clear_choice, write_folder)
+from helpers import collect, max_error, random_prompt, trace_mixed, trace_portions, trace_prefill_then_decode, trace_whole
+
+pytestmark = pytest.mark.gpu
+F64 = torch.float64
+# of the largest logit; bfloat16: rounding of the small widths, whose largest errors the plain-torch stand-in
+# of the kernels (the same places of rounding, other code) shows alike
+TOL = {"float32": 2e-5, "bfloat16": 4e-2}
+DTYPES = {"float32": torch.float32, "bfloat16": torch.bfloat16}
+
+
+@pytest.fixture(scope="module")
+def ops():
+    from tiny_llm_infer_amd.kernels.ops import HipOps
+    return HipOps("cuda:0")
+
+
+def _runner(folder, dtype, max_tokens, page, max_requests=4):
+    from tiny_llm_infer_amd.engine.loading import load_model
+    from tiny_llm_infer_amd.engine.runner import ModelRunner
+    model, _ = load_model(folder, dtype, "cuda:0", max_model_len=2048)
+    return ModelRunner(model, model.env, page_size=page, num_pages=max_tokens // page,
+                       max_requests=max_requests, max_batch_tokens=1024)
+
+
+def _replay(runner, steps):
+    from tiny_llm_infer_amd.engine.replay import Replayer
+    rp = Replayer(runner)
+    return {st["step"]: rp.run_step(st) for st in steps}
+
+
+def _requests(vocab, lengths, seed):
+    return {f"r{i}": random_prompt(vocab, n, seed + i) for i, n in enumerate(lengths)}
+
+
+def _close(got, want, tol, what):
+    got, want = got.detach().double().cpu(), want.double()
+    err, scale = float((got - want).abs().max()), float(want.abs().max())
+    assert err <= tol * max(scale, 1e-6), f"{what}: error {err:.3e}, scale {scale:.3e}"
+
+
+def _all_cuts(folder, dtype, reqs, want, page, max_tokens, tol, what):
+    cuts = {
+        "whole": trace_whole(reqs),
+        "decode": trace_prefill_then_decode(reqs),
+        "portions": trace_portions(reqs, seed=3),
+        "mixed": trace_mixed(reqs, max_tokens=max_tokens, seed=9),
+    }
+    for cut, steps in cuts.items():
+        runner = _runner(folder, dtype, max_tokens, page)
+        got = collect(steps, _replay(runner, steps))
+        for rid in reqs:
+            err, row, scale = max_error(got[rid], want[rid])
+            assert err <= tol * scale, f"{what}/{dtype}/{cut}/{rid}: error {err:.3e} at token {row} (scale {scale:.3e})"
+        runner.cache.check()
+        assert not runner.cache.live() and runner.cache.free_pages() == runner.cache.pages_per_group()
+        if cut == "mixed":
+            assert runner.cache.pages_taken_total > runner.cache.num_pages
+
+
+# ------------------------------------------------ the block's norm of what a sublayer gives ---
+@pytest.mark.parametrize("n", [72, 50, 1024, 4100])
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+def test_sublayer_output_normed_and_added(ops, dtype, n):
+    g = torch.Generator().manual_seed(n)
+    dt, T = DTYPES[dtype], 7
+    x = torch.randn(T, n, generator=g) * 3 + 1.5
+    y = (torch.randn(T, n, generator=g) * 5).to(dt)
+    y[3] = 0.0                                                       # a sublayer that gives nothing: eps alone under the root
+    w = torch.randn(n, generator=g) + 1
+    resid = x.clone().cuda()
+    rows = ops.norm_add(resid, y.cuda(), w.cuda(), 1e-5, dt)
+    want = x.double() + plain_gimipel.rms_norm(y.double(), w.double(), 1e-5)
+    _close(resid, want, 2e-6, "residual")
+    _close(rows, want, 2e-6 if dtype == "float32" else 4e-3, "rows handed on")
+    assert rows.dtype == dt and torch.equal(resid[3].cpu(), x[3])
+    first = ops.residual_rows(x.cuda(), dt)
+    assert first.dtype == dt and torch.equal(first.cpu(), x.to(dt))
+
+
+# ----------------------------------------------------------------- the router ---
+@pytest.mark.parametrize("outputs, top, groups, keep", [(6, 3, 3, 2), (4, 1, 1, 1), (8, 3, 8, 3), (16, 4, 4, 2), (12, 3, 2, 1),
+                                                        (64, 8, 8, 4), (5, 5, 1, 1)])
+def test_router_softmax_correction_and_groups_by_their_best(ops, outputs, top, groups, keep):
+    g = torch.Generator().manual_seed(outputs)
+    T = 41
+    z = torch.randn(T, outputs, generator=g) * 2
+    z[7] = -30.0
+    z[7, outputs - 1] = 10.0                                         # one output has it all: the others' choice scores are
+    corr = torch.randn(outputs, generator=g) * 0.2                   # their corrections, some below zero
+    w = {"router": torch.eye(outputs, dtype=F64), "correction": corr.double()}
+    f = {"router": {"experts": outputs - 1, "identity": 1, "top": top, "groups": {"count": groups, "keep": keep}}}
+    want_ids, want_wts = plain_gimipel.route(z.double(), f, w, "")
+    how = dict(score="softmax", group_score="max", normalize=False, correction=corr.cuda())
+    ids, wts, none = ops.route_experts(z.cuda(), outputs, top, groups, keep, 1.0, False, **how)
+    assert none is None and ids.cpu().tolist() == want_ids
+    _close(wts, torch.tensor(want_wts, dtype=F64), 1e-6, "weights")
+    ids2, wts2, _ = ops.route_experts(z.t().contiguous().cuda(), outputs, top, groups, keep, 1.0, False, transposed=True, **how)
+    assert torch.equal(ids2, ids) and torch.equal(wts2, wts)
+    del w["correction"]
+    want_ids, want_wts = plain_gimipel.route(z.double(), f, w, "")
+    how["correction"] = None
+    ids, wts, _ = ops.route_experts(z.cuda(), outputs, top, groups, keep, 1.0, False, **how)
+    assert ids.cpu().tolist() == want_ids
+    _close(wts, torch.tensor(want_wts, dtype=F64), 1e-6, "weights without a correction")
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16", "bfloat16-plain"])
+@pytest.mark.parametrize("T, E, ident, top, n, ff", [(1, 4, 1, 2, 48, 40), (5, 3, 3, 2, 64, 32), (40, 8, 2, 3, 104, 24),
+                                                     (300, 10, 4, 4, 128, 64), (130, 1, 2, 3, 136, 200)])
+def test_experts_that_hand_their_input_on(ops, dtype, T, E, ident, top, n, ff):
+    """Ids from E on stand for experts without matrices: their term is the weight times the row itself.  Rows
+    that choose only such experts, rows that choose none of them."""
+    g = torch.Generator().manual_seed(T)
+    dtype, _, variant = dtype.partition("-")
+    dt = DTYPES[dtype]
+    x = torch.randn(T, n, generator=g).to(dt)
+    w_gu = (torch.randn(E, 2 * ff, n, generator=g) * n ** -0.5).to(dt)
+    w_down = (torch.randn(E, n, ff, generator=g) * ff ** -0.5).to(dt)
+    ids = torch.stack([torch.randperm(E + ident, generator=g)[:top] for _ in range(T)]).to(torch.int32)
+    if ident >= top:
+        ids[0] = torch.arange(E, E + top)
+    wts = torch.rand(T, top, generator=g) + 0.2
+    shared = torch.randn(T, n, generator=g).to(dt)
+    want = shared.double().clone()
+    for t in range(T):
+        for j in range(top):
+            e = int(ids[t, j])
+            if e >= E:
+                want[t] += wts[t, j].double() * x[t].double()
+            else:
+                z = w_gu[e, :ff].double() @ x[t].double()
+                want[t] += wts[t, j].double() * (w_down[e].double() @ ((z * torch.sigmoid(z)) * (w_gu[e, ff:].double() @ x[t].double())))
+    packed = None if variant == "plain" else ops.pack_experts(w_gu.cuda(), w_down.cuda())
+    rowmajor = (None, None) if packed is not None else (w_gu.cuda(), w_down.cuda())
+    got = ops.apply_experts(x.cuda(), ids.cuda(), wts.cuda(), *rowmajor, packed, shared.cuda(), None)
+    _close(got, want, 2e-5 if dtype == "float32" else 2e-2, "experts, some of them without matrices, and the shared one")
+
+
+# ----------------------------------------------------- a matrix a head ---
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+@pytest.mark.parametrize("T, H, N, K, gap", [(1, 2, 16, 16, 0), (37, 3, 24, 40, 6), (200, 4, 96, 64, 32), (70, 2, 64, 512, 64),
+                                             (5, 16, 128, 128, 0), (33, 1, 48, 656, 8)])
+def test_product_with_a_matrix_of_its_own_for_every_head(ops, dtype, T, H, N, K, gap):
+    g = torch.Generator().manual_seed(T + N)
+    dt = DTYPES[dtype]
+    x = torch.randn(T, H * (K + gap) + 4, generator=g).to(dt)
+    w = (torch.randn(H, N, K, generator=g) * K ** -0.5).to(dt)
+    y = ops.head_products(x.cuda(), K + gap, w.cuda(), x_at=4)
+    heads = x[:, 4:].double().view(T, H, K + gap)[:, :, :K]
+    want = torch.einsum("thk,hnk->thn", heads, w.double()).reshape(T, H * N)
+    _close(y, want, 2e-6 if dtype == "float32" else 6e-3, "heads' products")
+    out = torch.full((T, H * (N + 8)), 3.0, dtype=dt, device="cuda")
+    ops.head_products(x.cuda(), K + gap, w.cuda(), out=out, out_stride=N + 8, x_at=4, out_at=8)
+    got = out.cpu().view(T, H, N + 8)
+    _close(got[:, :, 8:].reshape(T, H * N), want, 2e-6 if dtype == "float32" else 6e-3, "heads' products into a row with gaps")
+    assert float(got[:, :, :8].float().min()) == 3.0 == float(got[:, :, :8].float().max())   # nothing is written between them
+
+
+# --------------------------------------------------- one mixer alone, through the step function ---
+MIXERS = {
+    # two maps a head: sizes in sixteens (the matrix cores in bfloat16) and others, windows with and without kept keys
+    "two-maps 6/2 48/80 window 36+5": _attention(6, 2, 48, 80, 36, 5, diff=0.6),
+    "two-maps 8/1 32/16 window 21+0": _attention(8, 1, 32, 16, 21, 0, diff=0.2, scale=0.3),
+    "two-maps 3/3 20/12 no window": _attention(3, 3, 20, 12, None, 0, diff=0.7),
+    "two-maps 2/1 128/128 window 16+16": _attention(2, 1, 128, 128, 16, 16, diff=0.4),
+    "two-maps 34/2 16/16 window 70+1": _attention(34, 2, 16, 16, 70, 1, diff=0.5),
+    # one latent vector a position: part of the turned part turned, values longer than the latent vector
+    "latent 3 64+16 -> 96 of 80": _latent(3, 64, 16, 96, 80, base=1e6),
+    "latent 2 16+32(16) -> 16 of 48": _latent(2, 16, 32, 16, 48, base=100.0, dims=16),
+    "latent 5 24+6 -> 20 of 40": _latent(5, 24, 6, 20, 40),
+    "latent 20 32+16 -> 32 of 112": _latent(20, 32, 16, 32, 112),
+    "latent 1 128+64 -> 128 of 512": _latent(1, 128, 64, 128, 512),
+}
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+@pytest.mark.parametrize("name", list(MIXERS))
+def test_one_mixer_alone_in_every_cut(tmp_path, name, dtype):
+    """A model of one layer without feed-forward: the mixer's kernels (what they make of the projections, what they
+    write into the cache and read back, the heads' outputs) between an embedding and the head."""
+    mixer = MIXERS[name]
+    kind = "latent_attention" if "kv_rank" in mixer else "attention"
+    cfg = _config(120, 64 if mixer["heads"] < 20 else 96, [_layer(kind, mixer, None)], emb_scale=2.0)
+    folder = write_folder(str(tmp_path / "one"), cfg, make_weights(cfg, len(name), mild=dtype == "bfloat16"))
+    reqs = _requests(120, [70, 45, 137, 33, 1, 58, 2, 3], seed=5)
+    _all_cuts(folder, dtype, reqs, plain_logits(folder, reqs), 16, 384, TOL[dtype], name)
+
+
+# ---------------------------------------------- keys at the window's edges and at the kept ones' ---
+def _needle_model(tmp_path, window, keep_first, heads=2, dim=16, vdim=16):
+    """One layer of two-map attention whose keys are its queries (the same matrix and norm weights, as many key heads as
+    query heads) with a large score scale, so that a token's query finds the key of a like token among all
+    others.  Queries and keys read the first half of the width, values the second; tokens 88 and 89 have the same
+    first half: the query of 89 finds the key of 88 (beside its own), and the value there is another one."""
+    cfg = _config(90, 32, [_layer("attention", _attention(heads, heads, dim, vdim, window, keep_first, scale=1.5), None)], emb_scale=3.0)
+    w = {k: v.float() for k, v in make_weights(cfg, 4).items()}
+    w["l0.mix.q"][:, 16:] = 0.0
+    w["l0.mix.k"] = w["l0.mix.q"].clone()
+    w["l0.mix.k.norm"] = w["l0.mix.q.norm"].clone()
+    w["l0.mix.v"][:, :16] = 0.0
+    w["embed"][88, :16] = w["embed"][89, :16]
+    return cfg, write_folder(str(tmp_path / f"needle{window}_{keep_first}"), cfg, {k: v.to(torch.bfloat16) for k, v in w.items()})
+
+
+def _last_token_three_ways(folder, dtype, page, toks, want, what):
+    """The last token in a whole prompt, decoded alone, and at the end of a portion of two."""
+    from tiny_llm_infer_amd.engine.runner import StepEntry
+    n = len(toks)
+    for tail in (0, 1, 2):
+        runner = _runner(folder, dtype, 512, page)
+        runner.admit("x")
+        if tail:
+            runner.step([StepEntry("x", toks[:n - tail], [])])
+            got = runner.step([StepEntry("x", toks[n - tail:], [tail - 1])])
+        else:
+            got = runner.step([StepEntry("x", toks, [n - 1])])
+        err = np.abs(got[0].double().cpu().numpy() - want).max()
+        assert err <= TOL[dtype] * np.abs(want).max(), (what, tail, err)
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+@pytest.mark.parametrize("window, keep_first, page", [(24, 3, 16), (16, 16, 16), (33, 0, 8), (40, 17, 32), (5, 1, 16)])
+def test_one_key_that_stands_out_at_every_edge(tmp_path, dtype, window, keep_first, page):
+    """The token that the last query looks for stands window - 1 positions back (seen) or window positions back (not
+    seen), or far back at the last kept position (seen) or the one after it (not seen, though its page is still
+    held for the kept ones)."""
+    cfg, folder = _needle_model(tmp_path, window, keep_first)
+    w = plain_gimipel.read_model(folder)[1]
+    n = 3 * window + keep_first + 21
+    places = {"window_in": n - window, "window_out": n - 1 - window}
+    if keep_first:
+        places.update(first_in=keep_first - 1, first_out=keep_first)
+    logits = {}
+    for what, at in places.items():
+        toks = [t % 88 for t in random_prompt(88, n, 6)]              # neither id is in any of the other places
+        toks[at], toks[n - 1] = 88, 89
+        logits[what] = plain_gimipel.forward(cfg, w, toks)[-1].numpy()
+        _last_token_three_ways(folder, dtype, page, toks, logits[what], what)
+    # the test would not see an edge that is one off if the needle did not matter
+    assert np.abs(logits["window_in"] - logits["window_out"]).max() > 0.04 * np.abs(logits["window_out"]).max()
+    if keep_first:
+        assert np.abs(logits["first_in"] - logits["first_out"]).max() > 0.04 * np.abs(logits["first_out"]).max()
+        assert np.abs(logits["first_out"] - logits["window_out"]).max() < 1e-6 * np.abs(logits["window_out"]).max()
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+@pytest.mark.parametrize("heads, dim, rot, vdim, rank, page", [(2, 16, 8, 16, 24, 8), (4, 32, 16, 48, 64, 16)])
+def test_one_key_hundreds_of_positions_back(tmp_path, dtype, heads, dim, rot, vdim, rank, page):
+    """Latent attention sees everything: the query of the last token is made (by a change of rank one to the query
+    matrix) to point at what the latent vector of token 88 becomes as a key, and that token stands at position 2 of
+    430.  In a whole prompt, in portions, and with the last 40 tokens decoded one by one."""
+    cfg = _config(90, 32, [_layer("latent_attention", _latent(heads, dim, rot, vdim, rank, scale=1.0, base=100.0), None)], emb_scale=3.0)
+    w = {k: v.float() for k, v in make_weights(cfg, 9).items()}
+    eps = cfg["norm"]["eps"]
+    wq = w["l0.mix.q"].view(heads, dim + rot, 32)
+    wq[:, dim:] *= 0.05                                              # the turned parts say little
+    x_a, x_b = w["embed"][88].to(torch.bfloat16).float() * 3.0, w["embed"][89].to(torch.bfloat16).float() * 3.0
+    c = plain_gimipel.rms_norm((w["l0.mix.dkv"][:rank].to(torch.bfloat16).float() @ x_a).double(),
+                               w["l0.mix.dkv.norm"].to(torch.bfloat16).double(), eps).float()
+    key = (w["l0.mix.uk"].to(torch.bfloat16).float() @ c).view(heads, dim)
+    target = key * (30.0 / (key * key).sum(-1, keepdim=True))         # a score of 30 in every head
+    wq[:, :dim] += ((target - wq[:, :dim] @ x_b)[..., None] * x_b) / (x_b * x_b).sum()
+    folder = write_folder(str(tmp_path / "far"), cfg, {k: v.to(torch.bfloat16) for k, v in w.items()})
+    wd = plain_gimipel.read_model(folder)[1]
+    n = 430
+    toks = [t % 88 for t in random_prompt(88, n, 11)]
+    toks[n - 1] = 89
+    without = plain_gimipel.forward(cfg, wd, toks)[-1].numpy()
+    toks[2] = 88
+    want = plain_gimipel.forward(cfg, wd, toks)
+    assert np.abs(want[-1].numpy() - without).max() > 0.04 * np.abs(without).max()
+    _last_token_three_ways(folder, dtype, page, toks, want[-1].numpy(), "far")
+    reqs = {"r0": toks}
+    for steps in (trace_prefill_then_decode(reqs, tail=40), trace_portions(reqs, seed=5)):
+        got = collect(steps, _replay(_runner(folder, dtype, 448, page), steps))
+        # (bfloat16: the last row, whose softmax has one clear answer; the rows before it have scores as large and
+        # several keys that compete, which multiplies the rounding of the queries and keys)
+        first = 0 if dtype == "float32" else n - 1
+        err, row, scale = max_error(got["r0"][first:], want.numpy()[first:])
+        assert err <= TOL[dtype] * scale, (err, row)
+
+
+# ------------------------------------------------------------- the model, every cut ---
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+@pytest.mark.parametrize("name", list(SMALL))
+def test_all_cuts_match_plain(gimipel_folders, gimipel_clear_folders, name, dtype):
+    """float32: weights that are random throughout.  bfloat16: weights whose routers read nothing that rounding
+    touches, so that no close call is turned, and whose scores are smaller."""
+    folder = (gimipel_clear_folders if dtype == "bfloat16" else gimipel_folders)[name]
+    reqs = _requests(SMALL[name][0]["vocab"], [70, 45, 197, 33, 1, 58, 2, 3], seed=5)
+    if dtype == "bfloat16":
+        assert rows_with_a_clear_choice(folder, reqs, margin=1e-4) == {rid: len(t) for rid, t in reqs.items()}
+    _all_cuts(folder, dtype, reqs, plain_logits(folder, reqs), SMALL[name][1], 384, TOL[dtype], name)
+
+
+def test_token_by_token_from_the_first(gimipel_folders):
+    """Every token decoded alone from position 0: the first keys as they are written, the window as it starts to pass."""
+    for name in ("A", "K"):
+        folder = gimipel_folders[name]
+        reqs = _requests(SMALL[name][0]["vocab"], [60], seed=21)
+        want = plain_logits(folder, reqs)
+        steps = trace_prefill_then_decode(reqs, tail=59)
+        got = collect(steps, _replay(_runner(folder, "float32", 64, SMALL[name][1]), steps))
+        err, row, scale = max_error(got["r0"], want["r0"])
+        assert err <= TOL["float32"] * scale, (name, err, row)
+
+
+def test_unequal_requests_together_equal_each_alone(gimipel_folders):
+    """float32: a request's logits in a batch of unequal requests are those it has alone, to rounding."""
+    folder = gimipel_folders["R"]
+    reqs = _requests(320, [3, 130, 34, 65], seed=60)
+    alone = {rid: _replay(_runner(folder, "float32", 256, 32), trace_whole({rid: toks}))[0] for rid, toks in reqs.items()}
+    step = {"step": 0, "entries": [{"id": r, "tokens": t, "want": list(range(len(t)))} for r, t in reqs.items()], "end": list(reqs)}
+    together = collect([step], _replay(_runner(folder, "float32", 512, 32), [step]))
+    for rid in reqs:
+        assert np.abs(together[rid] - alone[rid]).max() <= 2e-5 * np.abs(alone[rid]).max()
+
+
+def test_long_decoding_through_recorded_launches(gimipel_clear_folders):
+    """150 tokens decoded one by one for three requests at once (bfloat16: the steps are replayed from
+    recordings), the window passing over decoded tokens and its pages given back on the way."""
+    folder = gimipel_clear_folders["R"]
+    reqs = _requests(320, [160, 171, 183], seed=77)
+    want = plain_logits(folder, reqs)
+    runner = _runner(folder, "bfloat16", 768, 32)
+    steps = [{"step": 0, "entries": [{"id": r, "tokens": t[:len(t) - 150], "want": []} for r, t in reqs.items()], "end": []}]
+    for j in range(150):
+        steps.append({"step": j + 1, "entries": [{"id": r, "tokens": [t[len(t) - 150 + j]], "want": [0]} for r, t in reqs.items()],
+                      "end": list(reqs) if j == 149 else []})
+    got = collect(steps, _replay(runner, steps))
+    assert runner.graph_replays > 100
+    for rid, toks in reqs.items():
+        err, row, scale = max_error(got[rid], want[rid][len(toks) - 150:])
+        assert err <= TOL["bfloat16"] * scale, (rid, err, row)
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+def test_greedy_generation_through_the_engine(gimipel_folders, gimipel_clear_folders, dtype):
+    from tiny_llm_infer_amd.engine.llm_engine import LLMEngine
+    from tiny_llm_infer_amd.sampling.params import SamplingParams
+    folder = (gimipel_clear_folders if dtype == "bfloat16" else gimipel_folders)["A"]
+    prompts = [random_prompt(160, n, 90 + n) for n in (4, 19, 30, 41)]
+    eng = LLMEngine.from_folder(folder, dtype=dtype, max_model_len=128, page_size=16, num_kv_blocks=32, max_num_seqs=3,
+                                max_num_batched_tokens=32)
+    got = eng.generate(prompts, SamplingParams(max_tokens=10, ignore_eos=True))
+    if dtype == "float32":
+        assert [r.token_ids for r in got] == [plain_greedy(folder, p, 10) for p in prompts]
+    else:
+        # rounding may turn a close call: every token must be the plain implementation's choice or within
+        # the rounding error of it, given the tokens before
+        cfg, w = plain_gimipel.read_model(folder)
+        for p, r in zip(prompts, got):
+            logits = plain_gimipel.forward(cfg, w, p + r.token_ids)[len(p) - 1:-1]
+            for z, t in zip(logits, r.token_ids):
+                assert float(z.max() - z[t]) <= 2 * TOL["bfloat16"] * float(z.abs().max())
+    eng.runner.cache.check()
+    assert eng.runner.cache.free_pages() == eng.runner.cache.pages_per_group()
+
+
+# ------------------------------------------------------------------ the command line ---
+def test_the_programs_take_a_gimipel_folder(gimipel_folders, tmp_path):
+    """bin/trace_run replays a mixed trace, model_main --infer generates greedily, and a model of random
+    weights made from a config.json alone loads and generates."""
+    root = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+    folder, vocab = gimipel_folders["C"], SMALL["C"][0]["vocab"]
+    reqs = _requests(vocab, [40, 9, 77, 23, 52], seed=12)
+    want = plain_logits(folder, reqs)
+    steps = trace_mixed(reqs, max_tokens=192, seed=4)
+    proc = subprocess.run([sys.executable, os.path.join(root, "bin", "trace_run"), "--model", folder, "--dtype", "float32",
+                           "--out", str(tmp_path / "out"), "--max-tokens", "192"],
+                          input="".join(json.dumps(s) + "\n" for s in steps), text=True, stdout=subprocess.PIPE,
+                          stderr=subprocess.PIPE, timeout=600)
+    assert proc.returncode == 0, proc.stderr[-2000:]
+    assert proc.stdout.split("\n")[:-1] == [f"done {s['step']}" for s in steps]
+    outputs = {s["step"]: np.fromfile(tmp_path / "out" / f"{s['step']}.f32", dtype="<f4").reshape(-1, vocab)
+               for s in steps if sum(len(e["want"]) for e in s["entries"])}
+    got = collect(steps, outputs)
+    for rid in reqs:
+        err, row, scale = max_error(got[rid], want[rid])
+        assert err <= TOL["float32"] * scale, (rid, err, row)
+    prompt = random_prompt(vocab, 21, 3)
+    proc = subprocess.run([sys.executable, os.path.join(root, "bin", "model_main"), "--infer", "--model", folder, "--dtype",
+                           "float32", "--prompt-ids", ",".join(map(str, prompt)), "--max-new-tokens", "8", "--ignore-eos",
+                           "--max-seq-len", "64", "--num-kv-blocks", "16"],
+                          text=True, stdout=subprocess.PIPE, stderr=subprocess.PIPE, timeout=600)
+    assert proc.returncode == 0, proc.stderr[-2000:]
+    assert [int(t) for t in proc.stdout.split()] == plain_greedy(folder, prompt, 8)
+    cfg_file = tmp_path / "config.json"
+    cfg_file.write_text(json.dumps(SMALL["R"][0]))
+    proc = subprocess.run([sys.executable, os.path.join(root, "bin", "model_main"), "--infer", "--config", str(cfg_file),
+                           "--random-weights", "--seed", "5", "--prompt-ids", "1,2,3,4,5", "--max-new-tokens", "6",
+                           "--ignore-eos", "--max-seq-len", "64", "--num-kv-blocks", "16"],
+                          text=True, stdout=subprocess.PIPE, stderr=subprocess.PIPE, timeout=600)
+    assert proc.returncode == 0, proc.stderr[-2000:]
+    assert len(proc.stdout.split()) == 6
