@@ -180,6 +180,8 @@ MIXERS = {
     "two-maps 3/3 20/12 no window": _attention(3, 3, 20, 12, None, 0, diff=0.7),
     "two-maps 2/1 128/128 window 16+16": _attention(2, 1, 128, 128, 16, 16, diff=0.4),
     "two-maps 34/2 16/16 window 70+1": _attention(34, 2, 16, 16, 70, 1, diff=0.5),
+    "two-maps 4/2 64/128 window 50+3": _attention(4, 2, 64, 128, 50, 3, diff=0.3),
+    "two-maps 2/2 128/256 window 30+2": _attention(2, 2, 128, 256, 30, 2, diff=0.5),
     # one latent vector a position: part of the turned part turned, values longer than the latent vector
     "latent 3 64+16 -> 96 of 80": _latent(3, 64, 16, 96, 80, base=1e6),
     "latent 2 16+32(16) -> 16 of 48": _latent(2, 16, 32, 16, 48, base=100.0, dims=16),
