@@ -1,23 +1,25 @@
-// Attention over the paged cache for heads whose keys and values have sizes of their own: the matrix-core kernel
-// for bfloat16, key and value sizes in sixteens.  It serves portions of prompts and single decoded rows alike.
-// What it computes is what attention_sized_plain.hip computes (maps of a head, values from a cache of their own or
-// the first elements of the keys, a window with kept first keys).
+// Attention over the paged cache for heads whose keys and values have sizes of their own: the matrix-core kernels
+// for bfloat16, key and value sizes in sixteens.  What they compute is what attention_sized_plain.hip computes
+// (maps of a head, values from a cache of their own or the first elements of the keys, a window with kept first
+// keys).  Two kernels:
 //
-// A workgroup of four waves takes 16 consecutive rows of one sequence (a "tile") and one (head, map); in steps of
-// single rows a tile is one row and its 16 columns are query heads that read the same key head (all heads, where
-// every head reads the one latent vector).  The keys a tile can see (from the first one its first row sees to its
-// last row, and the kept first ones before them) are walked 16 at a time, the waves taking every fourth 16 each with
-// a running maximum and sums of their own, merged through LDS at the end.  Every (row, key) pair is masked on its own.
+// attention_sized_shared_kernel (further down): portions of prompts, and single rows whose values are their keys'
+//   first elements (all heads read the one latent vector): four waves with 16 columns each share every tile of keys.
+// attention_sized_mfma_kernel (first): single decoded rows whose values have a cache of their own.  A workgroup of
+//   four waves takes one row and one (key head, map); its 16 columns are query heads that read that key head.  The keys
+//   the row can see (from the first one it sees to itself, and the kept first ones before them) are walked 16 at a
+//   time, the waves taking every fourth 16 each with a running maximum and sums of their own, merged through LDS at
+//   the end.  (It also takes tiles of 16 rows of a sequence and one head, as it did before the other kernel was there.)
 //
-// Everything is transposed: S^T = K Q^T and O^T = V^T P^T with v_mfma_f32_16x16x16_bf16, so that a row's scores lie in
-// the four lanes of a column and its weights are already the second operand of the output's product.  A wave brings
-// its 16 keys into LDS (16-byte loads, the next tile's in flight meanwhile) and reads the keys' fragments from there,
-// and the values' too where they are the keys' first elements; values with a cache of their own lie transposed
-// there ([dim][slot]), so that a lane's four keys of one dim are one 8-byte load from memory (a tile of 16 keys lies
-// inside one page: pages of 16 slots and more).
+// In both everything is transposed: S^T = K Q^T and O^T = V^T P^T with v_mfma_f32_16x16x16_bf16, so that a row's
+// scores lie in the four lanes of a column and its weights are already the second operand of the output's product.
+// Every (row, key) pair is masked on its own.  Keys come into LDS with 16-byte loads, the next tile's in flight
+// meanwhile, and their fragments are read from there; a value cache lies transposed ([dim][slot]), so that a lane's
+// four keys of one dim are 8 bytes (a tile of 16 keys lies inside one page: pages of 16 slots and more).
 //
-// The sizes are arguments, not template parameters: the registers for the query's fragments and the output's sums
-// are those of the largest size of a variant (keys up to 128 / 256 / 640 elements, values up to 128 / 256 / 512).
+// The sizes are arguments, not template parameters, but for the common sizes, which have kernels of their own (EXACT
+// below): the registers for the query's fragments and the output's sums are those of the largest size of a variant
+// (keys up to 128 / 256 / 640 elements, values up to 128 / 256 / 512).
 #include "common.h"
 
 typedef __attribute__((ext_vector_type(4))) short bf16x4;
@@ -326,7 +328,7 @@ __global__ __launch_bounds__(256) void attention_sized_shared_kernel(
     const bf16_t* __restrict__ q, TO* __restrict__ out, const bf16_t* __restrict__ k_cache,
     const bf16_t* __restrict__ v_cache, const int* __restrict__ row_start, const int* __restrict__ seq_start,
     int num_seqs, const int* __restrict__ tables, int table_width, int page_size, int num_pages, int heads,
-    int kv_heads, int maps, int nk_arg, int nv_arg, float scale, int window, int keep_first) {
+    int kv_heads, int maps, int nk_arg, int nv_arg, float scale, int window, int keep_first, int grouped) {
     const int nk = EXACT ? NKM : nk_arg, nv = EXACT ? NVM : nv_arg;
     const int DK = nk * 16, DV = nv * 16, LD = DK + ASM_PAD;
     const int pieces = 2 * nk;                                          // 16-byte pieces of one key
@@ -336,11 +338,14 @@ __global__ __launch_bounds__(256) void attention_sized_shared_kernel(
     const int tid = threadIdx.x, lane = tid % 64, wave = __builtin_amdgcn_readfirstlane(tid / 64);
     const int col = lane % 16, grp = lane / 16;
     const int per_kv = heads / kv_heads;
+    // grouped (steps of single rows): a column tile is one row, its columns 16 of the key head's query heads
+    const int per_tile = grouped ? 1 : 16;
+    const int cts_a_tile = grouped ? (per_kv + 15) / 16 : per_kv;       // column tiles that share a tile of rows
     int wg = blockIdx.x, seq = 0, first_row = 0, count = 0, n_ct = 0;
     for (; seq < num_seqs; ++seq) {
         first_row = row_start[seq];
         count = row_start[seq + 1] - first_row;
-        n_ct = ((count + 15) / 16) * per_kv;
+        n_ct = ((count + per_tile - 1) / per_tile) * cts_a_tile;
         const int n_wg = (n_ct + 3) / 4;
         if (wg < n_wg) break;
         wg -= n_wg;
@@ -350,25 +355,27 @@ __global__ __launch_bounds__(256) void attention_sized_shared_kernel(
     const int g = kh / maps;                                            // the values' head
     const int units = heads * maps;
     const int ct_last = min(wg * 4 + 3, n_ct - 1);
-    const int ct = min(wg * 4 + wave, n_ct - 1);                        // (a wave without a column tile repeats the last)
-    const bool stores = wg * 4 + wave < n_ct;
-    const int rt = ct / per_kv;
-    const int unit = (g * per_kv + ct % per_kv) * maps + kh % maps;
+    const int ct = min(wg * 4 + wave, n_ct - 1);
+    const bool stores = wg * 4 + wave < n_ct;                           // (a wave without a column tile only fetches)
+    const int rt = ct / cts_a_tile, hc = ct % cts_a_tile;
     const int base_pos = seq_start[seq];
     const int* table = tables + (size_t)seq * table_width;
     // the keys the workgroup's rows see: lo..hi and the kept first ones before them
-    const int rt_first = (wg * 4) / per_kv, rt_last = ct_last / per_kv;
-    const int hi = base_pos + min(count, rt_last * 16 + 16) - 1;
-    const int lo = window > 0 ? max(0, base_pos + rt_first * 16 - window + 1) : 0;
+    const int rt_first = (wg * 4) / cts_a_tile, rt_last = ct_last / cts_a_tile;
+    const int hi = base_pos + min(count, rt_last * per_tile + per_tile) - 1;
+    const int lo = window > 0 ? max(0, base_pos + rt_first * per_tile - window + 1) : 0;
     const int kept_hi = window > 0 ? min(keep_first, lo) : 0;
-    // this wave's rows
-    const int live = min(16, count - rt * 16);
-    const int my = min(col, live - 1);                                  // (idle columns repeat the last row; never stored)
-    const int row = first_row + rt * 16 + my;
-    const int qpos = base_pos + rt * 16 + my;
+    // this wave's rows and columns
+    const int live_rows = min(per_tile, count - rt * per_tile);
+    const int live = grouped ? min(16, per_kv - hc * 16) : live_rows;   // columns that are stored
+    const int my = grouped ? 0 : min(col, live - 1);                    // (idle columns repeat the last; never stored)
+    const int head = g * per_kv + (grouped ? hc * 16 + min(col, live - 1) : hc);
+    const int unit = head * maps + kh % maps;
+    const int row = first_row + rt * per_tile + my;
+    const int qpos = base_pos + rt * per_tile + my;
     const int qlo = window > 0 ? max(0, qpos - window + 1) : 0;
-    const int w_hi = base_pos + rt * 16 + live - 1;
-    const int w_lo = window > 0 ? max(0, base_pos + rt * 16 - window + 1) : 0;
+    const int w_hi = base_pos + rt * per_tile + live_rows - 1;
+    const int w_lo = window > 0 ? max(0, base_pos + rt * per_tile - window + 1) : 0;
     const size_t k_page = (size_t)kv_heads * maps * page_size * DK;
     const size_t v_page = (size_t)kv_heads * page_size * DV;
     const int page_shift = __builtin_ctz(page_size), page_mask = page_size - 1;
@@ -458,7 +465,7 @@ __global__ __launch_bounds__(256) void attention_sized_shared_kernel(
         if (more) fetch(tile_key(it + 1));
         const bf16_t* kt = lds + (size_t)(it & 1) * buf_elems;
         const bf16_t* vt = kt + (size_t)16 * LD;
-        if (k0 <= w_hi && (k0 + 15 >= w_lo || k0 < keep_first)) {       // (the same for the whole wave)
+        if (stores && k0 <= w_hi && (k0 + 15 >= w_lo || k0 < keep_first)) {   // (the same for the whole wave)
             // scores, transposed: A = the key k0 + col, this lane group's dims; two sums in turn, so that a matrix
             // instruction does not wait for the one before it
             f32x4 s = (f32x4){0.f, 0.f, 0.f, 0.f}, s_odd = (f32x4){0.f, 0.f, 0.f, 0.f};
@@ -554,10 +561,13 @@ extern "C" int tli_attention_sized_mfma_bf16(
     if (gy > 65535) return tli_fail("attention: %lld heads exceed the grid limit 65535", gy);
     hipStream_t s = (hipStream_t)stream;
     const int nk = key_dim / 16, nv = value_dim / 16;
-    if (!grouped) {
+    // Steps of single rows whose values have a cache of their own go to the kernel whose waves share out the keys
+    // (measured at 64 rows over 150 keys, 4 query heads a key head: 21 us against 28); everything else to the one
+    // whose waves share the tiles of keys.
+    if (!(grouped && v_cache)) {
         // (a sequence's column tiles are rounded up to whole workgroups: at most one more a sequence; a workgroup
         // without column tiles leaves)
-        const long long wgs = ((long long)tiles * per_kv + 3) / 4 + num_seqs;
+        const long long wgs = ((long long)tiles * (grouped ? col_groups : per_kv) + 3) / 4 + num_seqs;
         if (wgs > 0x7fffffffLL || kv_heads * maps > 65535) return tli_fail("attention: too many tiles for one launch");
         const dim3 sgrid((unsigned)wgs, (unsigned)(kv_heads * maps));
         const size_t sbytes = ast_lds_bytes(key_dim, value_dim);
@@ -573,7 +583,7 @@ extern "C" int tli_attention_sized_mfma_bf16(
         }                                                                                                                  \
         kernel<<<sgrid, 256, sbytes, s>>>((const bf16_t*)q, (TO*)out, (const bf16_t*)k_cache, (const bf16_t*)v_cache,      \
                                           row_start, seq_start, num_seqs, tables, table_width, page_size, num_pages,      \
-                                          heads, kv_heads, maps, nk, nv, scale, window, keep_first);                      \
+                                          heads, kv_heads, maps, nk, nv, scale, window, keep_first, grouped);             \
     }
 #define AST_SIZES(VKEY, TO)                                                   \
     if (nk <= 8 && nv <= 8) AST_ONE(8, 8, VKEY, TO, false)                    \
@@ -618,16 +628,11 @@ extern "C" int tli_attention_sized_mfma_bf16(
     if (nk <= 8 && nv <= 8) ASM_ONE(8, 8, VKEY, TO, false)                    \
     else if (nk <= 16 && nv <= 16) ASM_ONE(16, 16, VKEY, TO, false)           \
     else ASM_ONE(40, 32, VKEY, TO, false)
-    if (v_cache && out_f32 && nk == 4 && nv == 4) ASM_ONE(4, 4, false, float, true)
-    else if (v_cache && out_f32 && nk == 4 && nv == 8) ASM_ONE(4, 8, false, float, true)
-    else if (v_cache && out_f32 && nk == 8 && nv == 8) ASM_ONE(8, 8, false, float, true)
-    else if (v_cache && out_f32 && nk == 8 && nv == 16) ASM_ONE(8, 16, false, float, true)
-    else if (!v_cache && !out_f32 && nk == 36 && nv == 32) ASM_ONE(36, 32, true, bf16_t, true)
-    else if (v_cache) {
-        if (out_f32) { ASM_SIZES(false, float) } else { ASM_SIZES(false, bf16_t) }
-    } else {
-        if (out_f32) { ASM_SIZES(true, float) } else { ASM_SIZES(true, bf16_t) }
-    }
+    if (out_f32 && nk == 4 && nv == 4) ASM_ONE(4, 4, false, float, true)
+    else if (out_f32 && nk == 4 && nv == 8) ASM_ONE(4, 8, false, float, true)
+    else if (out_f32 && nk == 8 && nv == 8) ASM_ONE(8, 8, false, float, true)
+    else if (out_f32 && nk == 8 && nv == 16) ASM_ONE(8, 16, false, float, true)
+    else if (out_f32) { ASM_SIZES(false, float) } else { ASM_SIZES(false, bf16_t) }
 #undef ASM_SIZES
 #undef ASM_ONE
 #undef ASM_ARGS

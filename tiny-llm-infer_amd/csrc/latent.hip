@@ -136,36 +136,55 @@ union HpFrag {
     hp_bf16x4 v;
 };
 
-template <int KM>
+// A wave takes 16 rows (a workgroup 64, so that its four waves fetch the same blocks of W one after the other and
+// three of them find it in the cache) and walks all blocks of 16 outputs, two at a time with a sum each, so that a
+// matrix instruction does not wait for the one before it.  EXACT: K is 16 KM (no condition left in the loop over k).
+template <int KM, bool EXACT>
 __global__ __launch_bounds__(256) void head_products_mfma_kernel(const bf16_t* __restrict__ x, long long x_row, long long x_head,
                                                                  const bf16_t* __restrict__ w, bf16_t* __restrict__ y,
                                                                  long long y_row, long long y_head, int T, int N, int K) {
     const int lane = threadIdx.x % 64, wave = threadIdx.x / 64;
     const int col = lane % 16, grp = lane / 16;
-    const int t0 = blockIdx.x * 16, h = blockIdx.y;
+    const int t0 = (blockIdx.x * 4 + wave) * 16, h = blockIdx.y;
+    if (t0 >= T) return;                                                // (the whole wave; no barriers in this kernel)
     const int t = min(t0 + col, T - 1);                                 // (rows past the end repeat the last; never stored)
-    const int nk = K / 16;
+    const int nk = EXACT ? KM : K / 16;
     HpFrag xf[KM];
     const bf16_t* xr = x + (size_t)t * x_row + (size_t)h * x_head;
 #pragma unroll
-    for (int j = 0; j < KM; ++j)
+    for (int j = 0; j < KM; ++j) {
+        xf[j].u = make_uint2(0, 0);
         if (j < nk) xf[j].u = *reinterpret_cast<const uint2*>(xr + j * 16 + grp * 4);
-    for (int nb = wave; nb * 16 < N; nb += 4) {
-        const bf16_t* wr = w + ((size_t)h * N + nb * 16 + col) * K + grp * 4;
-        hp_f32x4 acc = (hp_f32x4){0.f, 0.f, 0.f, 0.f};
+    }
+    // (few rows: the blocks of outputs are shared out over blockIdx.z, an even number each)
+    const int per_z = (((N / 16 + gridDim.z - 1) / gridDim.z) + 1) & ~1;
+    const int nblocks = min(N / 16, (int)(blockIdx.z + 1) * per_z);
+    bf16_t* yr = y + (size_t)t * y_row + (size_t)h * y_head + grp * 4;
+    for (int nb = blockIdx.z * per_z; nb < nblocks; nb += 2) {
+        const bool two = nb + 1 < nblocks;
+        const bf16_t* wr0 = w + ((size_t)h * N + nb * 16 + col) * K + grp * 4;
+        const bf16_t* wr1 = two ? wr0 + (size_t)16 * K : wr0;
+        hp_f32x4 acc0 = (hp_f32x4){0.f, 0.f, 0.f, 0.f}, acc1 = (hp_f32x4){0.f, 0.f, 0.f, 0.f};
 #pragma unroll
         for (int j = 0; j < KM; ++j) {
             if (j < nk) {
-                HpFrag a;
-                a.u = *reinterpret_cast<const uint2*>(wr + j * 16);
-                acc = __builtin_amdgcn_mfma_f32_16x16x16bf16_1k(a.v, xf[j].v, acc, 0, 0, 0);
+                HpFrag a0, a1;
+                a0.u = *reinterpret_cast<const uint2*>(wr0 + j * 16);
+                a1.u = *reinterpret_cast<const uint2*>(wr1 + j * 16);
+                acc0 = __builtin_amdgcn_mfma_f32_16x16x16bf16_1k(a0.v, xf[j].v, acc0, 0, 0, 0);
+                acc1 = __builtin_amdgcn_mfma_f32_16x16x16bf16_1k(a1.v, xf[j].v, acc1, 0, 0, 0);
             }
         }
         if (t0 + col < T) {
             uint2 st;
-            st.x = pack_bf16x2(acc[0], acc[1]);
-            st.y = pack_bf16x2(acc[2], acc[3]);
-            *reinterpret_cast<uint2*>(y + (size_t)t * y_row + (size_t)h * y_head + nb * 16 + grp * 4) = st;
+            st.x = pack_bf16x2(acc0[0], acc0[1]);
+            st.y = pack_bf16x2(acc0[2], acc0[3]);
+            *reinterpret_cast<uint2*>(yr + nb * 16) = st;
+            if (two) {
+                st.x = pack_bf16x2(acc1[0], acc1[1]);
+                st.y = pack_bf16x2(acc1[2], acc1[3]);
+                *reinterpret_cast<uint2*>(yr + nb * 16 + 16) = st;
+            }
         }
     }
 }
@@ -181,13 +200,20 @@ extern "C" int tli_head_products_mfma_bf16(const void* x, long long x_row, long 
     if (heads <= 0 || heads > 65535 || !tli_head_products_mfma_takes(N, K, x_row, x_head, y_row, y_head))
         return tli_fail("head_products: the matrix-core kernel takes sizes in sixteens (k up to 640), not %d x %d", N, K);
     if ((((uintptr_t)x | (uintptr_t)w | (uintptr_t)y) & 7)) return tli_fail("head_products: operands must be 8-byte aligned");
-    const dim3 grid((rows + 15) / 16, heads);
+    const int row_groups = (rows + 63) / 64;
+    int shares = 512 / (row_groups * heads);                           // enough workgroups for the chip
+    shares = shares < 1 ? 1 : (shares > N / 32 ? (N / 32 < 1 ? 1 : N / 32) : shares);
+    const dim3 grid(row_groups, heads, shares);
     hipStream_t s = (hipStream_t)stream;
-    if (K <= 128)
-        head_products_mfma_kernel<8><<<grid, 256, 0, s>>>((const bf16_t*)x, x_row, x_head, (const bf16_t*)w, (bf16_t*)y, y_row, y_head,
-                                                         rows, N, K);
-    else
-        head_products_mfma_kernel<40><<<grid, 256, 0, s>>>((const bf16_t*)x, x_row, x_head, (const bf16_t*)w, (bf16_t*)y, y_row, y_head,
-                                                          rows, N, K);
+#define HP_ONE(KM, EXACT)                                                                                              \
+    head_products_mfma_kernel<KM, EXACT><<<grid, 256, 0, s>>>((const bf16_t*)x, x_row, x_head, (const bf16_t*)w, (bf16_t*)y, \
+                                                              y_row, y_head, rows, N, K)
+    if (K == 64) HP_ONE(4, true);
+    else if (K == 128) HP_ONE(8, true);
+    else if (K == 256) HP_ONE(16, true);
+    else if (K == 512) HP_ONE(32, true);
+    else if (K <= 128) HP_ONE(8, false);
+    else HP_ONE(40, false);
+#undef HP_ONE
     return tli_check_launch("head_products_mfma");
 }
