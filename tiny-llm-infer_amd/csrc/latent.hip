@@ -136,54 +136,67 @@ union HpFrag {
     hp_bf16x4 v;
 };
 
-// A wave takes 16 rows (a workgroup 64, so that its four waves fetch the same blocks of W one after the other and
-// three of them find it in the cache) and walks all blocks of 16 outputs, two at a time with a sum each, so that a
-// matrix instruction does not wait for the one before it.  EXACT: K is 16 KM (no condition left in the loop over k).
-template <int KM, bool EXACT>
+// A wave takes RT tiles of 16 rows and walks all blocks of 16 outputs, two at a time with a sum each, so that a
+// matrix instruction does not wait for the one before it; a block of W that it has fetched serves all its row tiles.
+// (A workgroup's four waves fetch the same blocks of W one after the other: three of them find it in the cache.)
+// EXACT: K is 16 KM (no condition left in the loop over k).
+template <int KM, bool EXACT, int RT>
 __global__ __launch_bounds__(256) void head_products_mfma_kernel(const bf16_t* __restrict__ x, long long x_row, long long x_head,
                                                                  const bf16_t* __restrict__ w, bf16_t* __restrict__ y,
                                                                  long long y_row, long long y_head, int T, int N, int K) {
     const int lane = threadIdx.x % 64, wave = threadIdx.x / 64;
     const int col = lane % 16, grp = lane / 16;
-    const int t0 = (blockIdx.x * 4 + wave) * 16, h = blockIdx.y;
+    const int t0 = (blockIdx.x * 4 + wave) * 16 * RT, h = blockIdx.y;
     if (t0 >= T) return;                                                // (the whole wave; no barriers in this kernel)
-    const int t = min(t0 + col, T - 1);                                 // (rows past the end repeat the last; never stored)
     const int nk = EXACT ? KM : K / 16;
-    HpFrag xf[KM];
-    const bf16_t* xr = x + (size_t)t * x_row + (size_t)h * x_head;
+    HpFrag xf[RT][KM];
 #pragma unroll
-    for (int j = 0; j < KM; ++j) {
-        xf[j].u = make_uint2(0, 0);
-        if (j < nk) xf[j].u = *reinterpret_cast<const uint2*>(xr + j * 16 + grp * 4);
+    for (int r = 0; r < RT; ++r) {
+        const int t = min(t0 + r * 16 + col, T - 1);                    // (rows past the end repeat the last; never stored)
+        const bf16_t* xr = x + (size_t)t * x_row + (size_t)h * x_head;
+#pragma unroll
+        for (int j = 0; j < KM; ++j) {
+            xf[r][j].u = make_uint2(0, 0);
+            if (j < nk) xf[r][j].u = *reinterpret_cast<const uint2*>(xr + j * 16 + grp * 4);
+        }
     }
     // (few rows: the blocks of outputs are shared out over blockIdx.z, an even number each)
     const int per_z = (((N / 16 + gridDim.z - 1) / gridDim.z) + 1) & ~1;
     const int nblocks = min(N / 16, (int)(blockIdx.z + 1) * per_z);
-    bf16_t* yr = y + (size_t)t * y_row + (size_t)h * y_head + grp * 4;
     for (int nb = blockIdx.z * per_z; nb < nblocks; nb += 2) {
         const bool two = nb + 1 < nblocks;
         const bf16_t* wr0 = w + ((size_t)h * N + nb * 16 + col) * K + grp * 4;
         const bf16_t* wr1 = two ? wr0 + (size_t)16 * K : wr0;
-        hp_f32x4 acc0 = (hp_f32x4){0.f, 0.f, 0.f, 0.f}, acc1 = (hp_f32x4){0.f, 0.f, 0.f, 0.f};
+        hp_f32x4 acc0[RT], acc1[RT];
+#pragma unroll
+        for (int r = 0; r < RT; ++r) acc0[r] = acc1[r] = (hp_f32x4){0.f, 0.f, 0.f, 0.f};
 #pragma unroll
         for (int j = 0; j < KM; ++j) {
             if (j < nk) {
                 HpFrag a0, a1;
                 a0.u = *reinterpret_cast<const uint2*>(wr0 + j * 16);
                 a1.u = *reinterpret_cast<const uint2*>(wr1 + j * 16);
-                acc0 = __builtin_amdgcn_mfma_f32_16x16x16bf16_1k(a0.v, xf[j].v, acc0, 0, 0, 0);
-                acc1 = __builtin_amdgcn_mfma_f32_16x16x16bf16_1k(a1.v, xf[j].v, acc1, 0, 0, 0);
+#pragma unroll
+                for (int r = 0; r < RT; ++r) {
+                    acc0[r] = __builtin_amdgcn_mfma_f32_16x16x16bf16_1k(a0.v, xf[r][j].v, acc0[r], 0, 0, 0);
+                    acc1[r] = __builtin_amdgcn_mfma_f32_16x16x16bf16_1k(a1.v, xf[r][j].v, acc1[r], 0, 0, 0);
+                }
             }
         }
-        if (t0 + col < T) {
-            uint2 st;
-            st.x = pack_bf16x2(acc0[0], acc0[1]);
-            st.y = pack_bf16x2(acc0[2], acc0[3]);
-            *reinterpret_cast<uint2*>(yr + nb * 16) = st;
-            if (two) {
-                st.x = pack_bf16x2(acc1[0], acc1[1]);
-                st.y = pack_bf16x2(acc1[2], acc1[3]);
-                *reinterpret_cast<uint2*>(yr + nb * 16 + 16) = st;
+#pragma unroll
+        for (int r = 0; r < RT; ++r) {
+            const int t = t0 + r * 16 + col;
+            if (t < T) {
+                bf16_t* yr = y + (size_t)t * y_row + (size_t)h * y_head + grp * 4 + nb * 16;
+                uint2 st;
+                st.x = pack_bf16x2(acc0[r][0], acc0[r][1]);
+                st.y = pack_bf16x2(acc0[r][2], acc0[r][3]);
+                *reinterpret_cast<uint2*>(yr) = st;
+                if (two) {
+                    st.x = pack_bf16x2(acc1[r][0], acc1[r][1]);
+                    st.y = pack_bf16x2(acc1[r][2], acc1[r][3]);
+                    *reinterpret_cast<uint2*>(yr + 16) = st;
+                }
             }
         }
     }
@@ -200,20 +213,23 @@ extern "C" int tli_head_products_mfma_bf16(const void* x, long long x_row, long 
     if (heads <= 0 || heads > 65535 || !tli_head_products_mfma_takes(N, K, x_row, x_head, y_row, y_head))
         return tli_fail("head_products: the matrix-core kernel takes sizes in sixteens (k up to 640), not %d x %d", N, K);
     if ((((uintptr_t)x | (uintptr_t)w | (uintptr_t)y) & 7)) return tli_fail("head_products: operands must be 8-byte aligned");
-    const int row_groups = (rows + 63) / 64;
+    // (many rows: a wave keeps 4 tiles of 16 rows, 2 where k is large, so that a block of W serves them all)
+    const int rt = rows < 1024 ? 1 : (K <= 128 ? 4 : (K <= 512 ? 2 : 1));
+    const int row_groups = (rows + 64 * rt - 1) / (64 * rt);
     int shares = 512 / (row_groups * heads);                           // enough workgroups for the chip
     shares = shares < 1 ? 1 : (shares > N / 32 ? (N / 32 < 1 ? 1 : N / 32) : shares);
     const dim3 grid(row_groups, heads, shares);
     hipStream_t s = (hipStream_t)stream;
-#define HP_ONE(KM, EXACT)                                                                                              \
-    head_products_mfma_kernel<KM, EXACT><<<grid, 256, 0, s>>>((const bf16_t*)x, x_row, x_head, (const bf16_t*)w, (bf16_t*)y, \
-                                                              y_row, y_head, rows, N, K)
-    if (K == 64) HP_ONE(4, true);
-    else if (K == 128) HP_ONE(8, true);
-    else if (K == 256) HP_ONE(16, true);
-    else if (K == 512) HP_ONE(32, true);
-    else if (K <= 128) HP_ONE(8, false);
-    else HP_ONE(40, false);
+#define HP_ONE(KM, EXACT, RT)                                                                                              \
+    head_products_mfma_kernel<KM, EXACT, RT><<<grid, 256, 0, s>>>((const bf16_t*)x, x_row, x_head, (const bf16_t*)w, (bf16_t*)y, \
+                                                                  y_row, y_head, rows, N, K)
+    if (K == 64) { if (rt == 4) HP_ONE(4, true, 4); else HP_ONE(4, true, 1); }
+    else if (K == 128) { if (rt == 4) HP_ONE(8, true, 4); else HP_ONE(8, true, 1); }
+    else if (K == 256) { if (rt == 2) HP_ONE(16, true, 2); else HP_ONE(16, true, 1); }
+    else if (K == 512) { if (rt == 2) HP_ONE(32, true, 2); else HP_ONE(32, true, 1); }
+    else if (K <= 128) { if (rt == 4) HP_ONE(8, false, 4); else HP_ONE(8, false, 1); }
+    else if (K <= 512) { if (rt == 2) HP_ONE(32, false, 2); else HP_ONE(32, false, 1); }
+    else HP_ONE(40, false, 1);
 #undef HP_ONE
     return tli_check_launch("head_products_mfma");
 }
