@@ -323,8 +323,8 @@ static inline size_t ast_lds_bytes(int DK, int DV) {
     return 2 * ((size_t)16 * (DK + ASM_PAD) + (size_t)DV * AST_VLD) * 2;
 }
 
-template <int NKM, int NVM, bool VKEY, typename TO, bool EXACT>
-__global__ __launch_bounds__(256) void attention_sized_shared_kernel(
+template <int NKM, int NVM, bool VKEY, typename TO, bool EXACT, int WAVES>
+__global__ __launch_bounds__(64 * WAVES) void attention_sized_shared_kernel(
     const bf16_t* __restrict__ q, TO* __restrict__ out, const bf16_t* __restrict__ k_cache,
     const bf16_t* __restrict__ v_cache, const int* __restrict__ row_start, const int* __restrict__ seq_start,
     int num_seqs, const int* __restrict__ tables, int table_width, int page_size, int num_pages, int heads,
@@ -332,8 +332,8 @@ __global__ __launch_bounds__(256) void attention_sized_shared_kernel(
     const int nk = EXACT ? NKM : nk_arg, nv = EXACT ? NVM : nv_arg;
     const int DK = nk * 16, DV = nv * 16, LD = DK + ASM_PAD;
     const int pieces = 2 * nk;                                          // 16-byte pieces of one key
-    constexpr int KPASS = (2 * NKM + 15) / 16;                          // pieces of its key a thread brings
-    constexpr int VPASS = VKEY ? 1 : (32 * NVM + 255) / 256;            // 16-byte pieces of V^T a thread brings
+    constexpr int KPASS = (2 * NKM + 4 * WAVES - 1) / (4 * WAVES);                          // pieces of its key a thread brings
+    constexpr int VPASS = VKEY ? 1 : (32 * NVM + 64 * WAVES - 1) / (64 * WAVES);            // 16-byte pieces of V^T a thread brings
     extern __shared__ __align__(16) unsigned char ast_lds[];
     const int tid = threadIdx.x, lane = tid % 64, wave = __builtin_amdgcn_readfirstlane(tid / 64);
     const int col = lane % 16, grp = lane / 16;
@@ -346,22 +346,27 @@ __global__ __launch_bounds__(256) void attention_sized_shared_kernel(
         first_row = row_start[seq];
         count = row_start[seq + 1] - first_row;
         n_ct = ((count + per_tile - 1) / per_tile) * cts_a_tile;
-        const int n_wg = (n_ct + 3) / 4;
-        if (wg < n_wg) break;
+        const int n_wg = (n_ct + WAVES - 1) / WAVES;
+        if (wg < n_wg) {
+            // a sequence's last rows see the most keys: their workgroups start first, and the short ones fill in
+            // behind them as compute units come free
+            wg = n_wg - 1 - wg;
+            break;
+        }
         wg -= n_wg;
     }
     if (seq >= num_seqs) return;                                        // (the whole workgroup)
     const int kh = blockIdx.y;                                          // key head * maps + map
     const int g = kh / maps;                                            // the values' head
     const int units = heads * maps;
-    const int ct_last = min(wg * 4 + 3, n_ct - 1);
-    const int ct = min(wg * 4 + wave, n_ct - 1);
-    const bool stores = wg * 4 + wave < n_ct;                           // (a wave without a column tile only fetches)
+    const int ct_last = min(wg * WAVES + WAVES - 1, n_ct - 1);
+    const int ct = min(wg * WAVES + wave, n_ct - 1);
+    const bool stores = wg * WAVES + wave < n_ct;                           // (a wave without a column tile only fetches)
     const int rt = ct / cts_a_tile, hc = ct % cts_a_tile;
     const int base_pos = seq_start[seq];
     const int* table = tables + (size_t)seq * table_width;
     // the keys the workgroup's rows see: lo..hi and the kept first ones before them
-    const int rt_first = (wg * 4) / cts_a_tile, rt_last = ct_last / cts_a_tile;
+    const int rt_first = (wg * WAVES) / cts_a_tile, rt_last = ct_last / cts_a_tile;
     const int hi = base_pos + min(count, rt_last * per_tile + per_tile) - 1;
     const int lo = window > 0 ? max(0, base_pos + rt_first * per_tile - window + 1) : 0;
     const int kept_hi = window > 0 ? min(keep_first, lo) : 0;
@@ -413,7 +418,7 @@ __global__ __launch_bounds__(256) void attention_sized_shared_kernel(
         const bf16_t* src = k_cache + (size_t)(there ? page : 0) * k_page + ((size_t)kh * page_size + ((k0 + kk) & page_mask)) * DK;
 #pragma unroll
         for (int ps = 0; ps < KPASS; ++ps) {
-            const int p = ps * 16 + p0;
+            const int p = ps * (4 * WAVES) + p0;
             next_k[ps] = make_uint4(0, 0, 0, 0);
             if (there && p < pieces) next_k[ps] = *reinterpret_cast<const uint4*>(src + p * 8);
         }
@@ -421,7 +426,7 @@ __global__ __launch_bounds__(256) void attention_sized_shared_kernel(
             const bf16_t* vsrc = v_cache + (size_t)(there ? page : 0) * v_page + (size_t)g * DV * page_size + (k0 & page_mask);
 #pragma unroll
             for (int ps = 0; ps < VPASS; ++ps) {
-                const int c = ps * 256 + tid;                           // dim c / 2, keys 8 (c % 2) .. + 7 of the tile
+                const int c = ps * (64 * WAVES) + tid;                           // dim c / 2, keys 8 (c % 2) .. + 7 of the tile
                 next_v[ps] = make_uint4(0, 0, 0, 0);
                 if (there && c < 2 * DV) next_v[ps] = *reinterpret_cast<const uint4*>(vsrc + (size_t)(c >> 1) * page_size + (c & 1) * 8);
             }
@@ -432,7 +437,7 @@ __global__ __launch_bounds__(256) void attention_sized_shared_kernel(
         bf16_t* vt = buf + (size_t)16 * LD;
 #pragma unroll
         for (int ps = 0; ps < KPASS; ++ps) {
-            const int p = ps * 16 + p0;
+            const int p = ps * (4 * WAVES) + p0;
             if (p < pieces) {
                 *reinterpret_cast<uint4*>(kt + kk * LD + p * 8) = next_k[ps];
                 if (VKEY && p * 8 < DV) {
@@ -446,7 +451,7 @@ __global__ __launch_bounds__(256) void attention_sized_shared_kernel(
         if (!VKEY) {
 #pragma unroll
             for (int ps = 0; ps < VPASS; ++ps) {
-                const int c = ps * 256 + tid;
+                const int c = ps * (64 * WAVES) + tid;
                 if (c < 2 * DV) {
                     bf16_t* dst = vt + (c >> 1) * AST_VLD + (c & 1) * 8;    // (8-byte aligned, not 16)
                     *reinterpret_cast<uint2*>(dst) = make_uint2(next_v[ps].x, next_v[ps].y);
@@ -567,13 +572,16 @@ extern "C" int tli_attention_sized_mfma_bf16(
     if (!(grouped && v_cache)) {
         // (a sequence's column tiles are rounded up to whole workgroups: at most one more a sequence; a workgroup
         // without column tiles leaves)
-        const long long wgs = ((long long)tiles * (grouped ? col_groups : per_kv) + 3) / 4 + num_seqs;
+        // (eight waves a workgroup, two a SIMD, for portions of prompts over the large latent vector, where that
+        // still leaves two workgroups and more a compute unit to even out the rows that see few keys)
+        const int waves = (!grouped && !v_cache && !out_f32 && nk == 36 && nv == 32 && (long long)tiles * per_kv >= 8 * 512) ? 8 : 4;
+        const long long wgs = ((long long)tiles * (grouped ? col_groups : per_kv) + waves - 1) / waves + num_seqs;
         if (wgs > 0x7fffffffLL || kv_heads * maps > 65535) return tli_fail("attention: too many tiles for one launch");
         const dim3 sgrid((unsigned)wgs, (unsigned)(kv_heads * maps));
         const size_t sbytes = ast_lds_bytes(key_dim, value_dim);
-#define AST_ONE(NKM, NVM, VKEY, TO, EXACT)                                                                                        \
+#define AST_ONE(NKM, NVM, VKEY, TO, EXACT, WAVES)                                                                                        \
     {                                                                                                                      \
-        auto kernel = attention_sized_shared_kernel<NKM, NVM, VKEY, TO, EXACT>;                                                   \
+        auto kernel = attention_sized_shared_kernel<NKM, NVM, VKEY, TO, EXACT, WAVES>;                                                   \
         static bool allowed = false;                                                                                       \
         if (sbytes > 65536 && !allowed) {                                                                                  \
             if (hipFuncSetAttribute((const void*)kernel, hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024) !=        \
@@ -581,21 +589,22 @@ extern "C" int tli_attention_sized_mfma_bf16(
                 return tli_fail("attention: cannot have %zu bytes of LDS", sbytes);                                        \
             allowed = true;                                                                                                \
         }                                                                                                                  \
-        kernel<<<sgrid, 256, sbytes, s>>>((const bf16_t*)q, (TO*)out, (const bf16_t*)k_cache, (const bf16_t*)v_cache,      \
+        kernel<<<sgrid, 64 * WAVES, sbytes, s>>>((const bf16_t*)q, (TO*)out, (const bf16_t*)k_cache, (const bf16_t*)v_cache,      \
                                           row_start, seq_start, num_seqs, tables, table_width, page_size, num_pages,      \
                                           heads, kv_heads, maps, nk, nv, scale, window, keep_first, grouped);             \
     }
 #define AST_SIZES(VKEY, TO)                                                   \
-    if (nk <= 8 && nv <= 8) AST_ONE(8, 8, VKEY, TO, false)                    \
-    else if (nk <= 16 && nv <= 16) AST_ONE(16, 16, VKEY, TO, false)           \
-    else AST_ONE(40, 32, VKEY, TO, false)
+    if (nk <= 8 && nv <= 8) AST_ONE(8, 8, VKEY, TO, false, 4)                 \
+    else if (nk <= 16 && nv <= 16) AST_ONE(16, 16, VKEY, TO, false, 4)        \
+    else AST_ONE(40, 32, VKEY, TO, false, 4)
         // (sizes with a kernel of their own: heads of 64 and 128 with values of 64 to 256 in float32, for the
         // attention with two maps; a latent vector of 512 beside a turned part of 64)
-        if (v_cache && out_f32 && nk == 4 && nv == 4) AST_ONE(4, 4, false, float, true)
-        else if (v_cache && out_f32 && nk == 4 && nv == 8) AST_ONE(4, 8, false, float, true)
-        else if (v_cache && out_f32 && nk == 8 && nv == 8) AST_ONE(8, 8, false, float, true)
-        else if (v_cache && out_f32 && nk == 8 && nv == 16) AST_ONE(8, 16, false, float, true)
-        else if (!v_cache && !out_f32 && nk == 36 && nv == 32) AST_ONE(36, 32, true, bf16_t, true)
+        if (v_cache && out_f32 && nk == 4 && nv == 4) AST_ONE(4, 4, false, float, true, 4)
+        else if (v_cache && out_f32 && nk == 4 && nv == 8) AST_ONE(4, 8, false, float, true, 4)
+        else if (v_cache && out_f32 && nk == 8 && nv == 8) AST_ONE(8, 8, false, float, true, 4)
+        else if (v_cache && out_f32 && nk == 8 && nv == 16) AST_ONE(8, 16, false, float, true, 4)
+        else if (waves == 8) AST_ONE(36, 32, true, bf16_t, true, 8)
+        else if (!v_cache && !out_f32 && nk == 36 && nv == 32) AST_ONE(36, 32, true, bf16_t, true, 4)
         else if (v_cache) {
             if (out_f32) { AST_SIZES(false, float) } else { AST_SIZES(false, bf16_t) }
         } else {
