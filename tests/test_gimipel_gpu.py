@@ -183,12 +183,17 @@ MIXERS = {
     "two-maps 34/2 16/16 window 70+1": _attention(34, 2, 16, 16, 70, 1, diff=0.5),
     "two-maps 4/2 64/128 window 50+3": _attention(4, 2, 64, 128, 50, 3, diff=0.3),
     "two-maps 2/2 128/256 window 30+2": _attention(2, 2, 128, 256, 30, 2, diff=0.5),
+    # (sizes in sixteens without kernels of their own: the variants whose sizes are arguments)
+    "two-maps 2/1 160/48 window 25+6": _attention(2, 1, 160, 48, 25, 6, diff=0.4),
+    "two-maps 2/2 32/272 window 45+2": _attention(2, 2, 32, 272, 45, 2, diff=0.6),
     # one latent vector a position: part of the turned part turned, values longer than the latent vector
     "latent 3 64+16 -> 96 of 80": _latent(3, 64, 16, 96, 80, base=1e6),
     "latent 2 16+32(16) -> 16 of 48": _latent(2, 16, 32, 16, 48, base=100.0, dims=16),
     "latent 5 24+6 -> 20 of 40": _latent(5, 24, 6, 20, 40),
     "latent 20 32+16 -> 32 of 112": _latent(20, 32, 16, 32, 112),
     "latent 1 128+64 -> 128 of 512": _latent(1, 128, 64, 128, 512),
+    "latent 2 32+16 -> 48 of 144": _latent(2, 32, 16, 48, 144),
+    "latent 3 64+32 -> 64 of 320": _latent(3, 64, 32, 64, 320),
 }
 
 
