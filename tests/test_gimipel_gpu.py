@@ -156,7 +156,8 @@ def test_experts_that_hand_their_input_on(ops, dtype, T, E, ident, top, n, ff):
 @pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
 @pytest.mark.parametrize("T, H, N, K, gap", [(1, 2, 16, 16, 0), (37, 3, 24, 40, 6), (200, 4, 96, 64, 32), (70, 2, 64, 512, 64),
                                              (5, 16, 128, 128, 0), (33, 1, 48, 656, 8), (1100, 2, 32, 128, 0),
-                                             (1040, 2, 48, 512, 16), (1030, 1, 16, 80, 0), (1025, 3, 80, 272, 0)])
+                                             (1040, 2, 48, 512, 16), (1030, 1, 16, 80, 0), (1025, 3, 80, 272, 0),
+                                             (1024, 2, 80, 64, 8), (1200, 1, 144, 256, 0), (2048, 3, 512, 128, 32)])
 def test_product_with_a_matrix_of_its_own_for_every_head(ops, dtype, T, H, N, K, gap):
     g = torch.Generator().manual_seed(T + N)
     dt = DTYPES[dtype]

@@ -202,6 +202,91 @@ __global__ __launch_bounds__(256) void head_products_mfma_kernel(const bf16_t* _
     }
 }
 
+// Many rows, k of 64, 128, 256 or 512: the head's matrix comes through LDS.  A workgroup takes one head and 64 RT rows
+// (a wave RT tiles of 16, their fragments in registers) and walks the outputs in chunks of 8192 elements of W (NB
+// blocks of 16 outputs), which its 256 threads bring into one of two LDS buffers with 16-byte loads while the chunk
+// before is multiplied; the waves read the blocks' fragments from there (rows of k + 8 elements: 8-byte reads without
+// bank conflicts), each fragment serving the wave's RT row tiles, with two sums a row tile taking turns.
+template <int KM, int RT>
+__global__ __launch_bounds__(256) void head_products_lds_kernel(const bf16_t* __restrict__ x, long long x_row, long long x_head,
+                                                                const bf16_t* __restrict__ w, bf16_t* __restrict__ y,
+                                                                long long y_row, long long y_head, int T, int N) {
+    constexpr int K = KM * 16, LDW = K + 8, NB = 32 / KM, ROWS = NB * 16, PIECES = K / 8;
+    __shared__ __align__(16) bf16_t wt[2][ROWS * LDW];
+    const int tid = threadIdx.x, lane = tid % 64, wave = tid / 64;
+    const int col = lane % 16, grp = lane / 16;
+    const int t0 = (blockIdx.x * 4 + wave) * 16 * RT, h = blockIdx.y;
+    HpFrag xf[RT][KM];
+#pragma unroll
+    for (int r = 0; r < RT; ++r) {
+        const int t = min(t0 + r * 16 + col, T - 1);                    // (rows past the end repeat the last; never stored)
+        const bf16_t* xr = x + (size_t)t * x_row + (size_t)h * x_head;
+#pragma unroll
+        for (int j = 0; j < KM; ++j) xf[r][j].u = *reinterpret_cast<const uint2*>(xr + j * 16 + grp * 4);
+    }
+    const bf16_t* wh = w + (size_t)h * N * K;
+    const int chunks = (N + ROWS - 1) / ROWS;
+    uint4 next[4];                                                      // ROWS * PIECES = 1024 pieces of 16 bytes a chunk
+    auto fetch = [&](int c) {
+#pragma unroll
+        for (int i = 0; i < 4; ++i) {
+            const int idx = i * 256 + tid;
+            const int n = c * ROWS + idx / PIECES;
+            next[i] = make_uint4(0, 0, 0, 0);
+            if (n < N) next[i] = *reinterpret_cast<const uint4*>(wh + (size_t)n * K + (idx % PIECES) * 8);
+        }
+    };
+    auto store = [&](bf16_t* buf) {
+#pragma unroll
+        for (int i = 0; i < 4; ++i) {
+            const int idx = i * 256 + tid;
+            *reinterpret_cast<uint4*>(buf + (idx / PIECES) * LDW + (idx % PIECES) * 8) = next[i];
+        }
+    };
+    fetch(0);
+    store(wt[0]);
+    __syncthreads();
+    for (int c = 0; c < chunks; ++c) {
+        const bool more = c + 1 < chunks;
+        if (more) fetch(c + 1);
+        const bf16_t* buf = wt[c & 1];
+#pragma unroll
+        for (int nb = 0; nb < NB; ++nb) {
+            hp_f32x4 even[RT], odd[RT];
+#pragma unroll
+            for (int r = 0; r < RT; ++r) even[r] = odd[r] = (hp_f32x4){0.f, 0.f, 0.f, 0.f};
+            const bf16_t* wr = buf + (nb * 16 + col) * LDW + grp * 4;
+#pragma unroll
+            for (int j = 0; j < KM; ++j) {
+                HpFrag a;
+                a.u = *reinterpret_cast<const uint2*>(wr + j * 16);
+#pragma unroll
+                for (int r = 0; r < RT; ++r) {
+                    if (j % 2)
+                        odd[r] = __builtin_amdgcn_mfma_f32_16x16x16bf16_1k(a.v, xf[r][j].v, odd[r], 0, 0, 0);
+                    else
+                        even[r] = __builtin_amdgcn_mfma_f32_16x16x16bf16_1k(a.v, xf[r][j].v, even[r], 0, 0, 0);
+                }
+            }
+            const int n0 = (c * NB + nb) * 16;
+            if (n0 < N) {
+#pragma unroll
+                for (int r = 0; r < RT; ++r) {
+                    const int t = t0 + r * 16 + col;
+                    if (t < T) {
+                        uint2 st;
+                        st.x = pack_bf16x2(even[r][0] + odd[r][0], even[r][1] + odd[r][1]);
+                        st.y = pack_bf16x2(even[r][2] + odd[r][2], even[r][3] + odd[r][3]);
+                        *reinterpret_cast<uint2*>(y + (size_t)t * y_row + (size_t)h * y_head + n0 + grp * 4) = st;
+                    }
+                }
+            }
+        }
+        if (more) store(wt[(c + 1) & 1]);
+        __syncthreads();                                // the next chunk is written; this one is read by all
+    }
+}
+
 extern "C" int tli_head_products_mfma_takes(int N, int K, long long x_row, long long x_head, long long y_row, long long y_head) {
     return (N % 16 == 0 && K % 16 == 0 && N >= 16 && K >= 16 && K <= 640 && x_row % 4 == 0 && x_head % 4 == 0 &&
             y_row % 4 == 0 && y_head % 4 == 0) ? 1 : 0;
@@ -213,6 +298,19 @@ extern "C" int tli_head_products_mfma_bf16(const void* x, long long x_row, long 
     if (heads <= 0 || heads > 65535 || !tli_head_products_mfma_takes(N, K, x_row, x_head, y_row, y_head))
         return tli_fail("head_products: the matrix-core kernel takes sizes in sixteens (k up to 640), not %d x %d", N, K);
     if ((((uintptr_t)x | (uintptr_t)w | (uintptr_t)y) & 7)) return tli_fail("head_products: operands must be 8-byte aligned");
+    if (rows >= 1024 && (K == 64 || K == 128 || K == 256 || K == 512)) {
+        const dim3 lgrid((rows + 127) / 128, heads);
+        hipStream_t ls = (hipStream_t)stream;
+#define HP_LDS(KM)                                                                                                       \
+    head_products_lds_kernel<KM, 2><<<lgrid, 256, 0, ls>>>((const bf16_t*)x, x_row, x_head, (const bf16_t*)w, (bf16_t*)y, \
+                                                           y_row, y_head, rows, N)
+        if (K == 64) HP_LDS(4);
+        else if (K == 128) HP_LDS(8);
+        else if (K == 256) HP_LDS(16);
+        else HP_LDS(32);
+#undef HP_LDS
+        return tli_check_launch("head_products_lds");
+    }
     // (many rows: a wave keeps 4 tiles of 16 rows, 2 where k is large, so that a block of W serves them all)
     const int rt = rows < 1024 ? 1 : (K <= 128 ? 4 : (K <= 512 ? 2 : 1));
     const int row_groups = (rows + 64 * rt - 1) / (64 * rt);
