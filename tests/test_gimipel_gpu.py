@@ -252,9 +252,9 @@ def test_one_key_that_stands_out_at_every_edge(tmp_path, dtype, window, keep_fir
     cfg, folder = _needle_model(tmp_path, window, keep_first)
     w = plain_gimipel.read_model(folder)[1]
     n = 3 * window + keep_first + 21
-    places = {"window_in": n - window, "window_out": n - 1 - window}
+    places = {"inside_window": n - window, "outside_window": n - 1 - window}
     if keep_first:
-        places.update(first_in=keep_first - 1, first_out=keep_first)
+        places.update(last_kept=keep_first - 1, past_kept=keep_first)
     logits = {}
     for what, at in places.items():
         toks = [t % 88 for t in random_prompt(88, n, 6)]              # neither id is in any of the other places
@@ -262,10 +262,10 @@ def test_one_key_that_stands_out_at_every_edge(tmp_path, dtype, window, keep_fir
         logits[what] = plain_gimipel.forward(cfg, w, toks)[-1].numpy()
         _last_token_three_ways(folder, dtype, page, toks, logits[what], what)
     # the test would not see an edge that is one off if the needle did not matter
-    assert np.abs(logits["window_in"] - logits["window_out"]).max() > 0.04 * np.abs(logits["window_out"]).max()
+    assert np.abs(logits["inside_window"] - logits["outside_window"]).max() > 0.04 * np.abs(logits["outside_window"]).max()
     if keep_first:
-        assert np.abs(logits["first_in"] - logits["first_out"]).max() > 0.04 * np.abs(logits["first_out"]).max()
-        assert np.abs(logits["first_out"] - logits["window_out"]).max() < 1e-6 * np.abs(logits["window_out"]).max()
+        assert np.abs(logits["last_kept"] - logits["past_kept"]).max() > 0.04 * np.abs(logits["past_kept"]).max()
+        assert np.abs(logits["past_kept"] - logits["outside_window"]).max() < 1e-6 * np.abs(logits["outside_window"]).max()
 
 
 @pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
