@@ -211,6 +211,31 @@ def test_one_mixer_alone_in_every_cut(tmp_path, name, dtype):
     _all_cuts(folder, dtype, reqs, plain_logits(folder, reqs), 16, 384, TOL[dtype], name)
 
 
+def test_a_long_prompt_of_many_heads_over_the_large_latent_vector(tmp_path):
+    """2,048 rows of 32 heads over a latent vector of 512 beside a turned part of 64, in one step: enough column
+    tiles for the variant of the attention kernel with eight waves a workgroup; then the same prompt in two steps."""
+    from tiny_llm_infer_amd.engine.loading import load_model
+    from tiny_llm_infer_amd.engine.runner import ModelRunner, StepEntry
+    cfg = _config(150, 64, [_layer("latent_attention", _latent(32, 16, 64, 16, 512, base=1e4, dims=32), None)], emb_scale=2.0)
+    folder = write_folder(str(tmp_path / "long"), cfg, make_weights(cfg, 17, mild=True))
+    toks = random_prompt(150, 2048, 31)
+    want = plain_gimipel.forward(*plain_gimipel.read_model(folder), toks).numpy()
+    rows = [0, 1, 15, 16, 17, 500, 1023, 1024, 1025, 2000, 2046, 2047]
+    for cuts in ([2048], [1029, 1019]):
+        model, _ = load_model(folder, "bfloat16", "cuda:0", max_model_len=2048)
+        runner = ModelRunner(model, model.env, page_size=16, num_pages=130, max_requests=2, max_batch_tokens=2048)
+        runner.admit("x")
+        at = 0
+        for n in cuts:
+            here = [r - at for r in rows if at <= r < at + n]
+            got = runner.step([StepEntry("x", toks[at:at + n], here)]).double().cpu().numpy()
+            ref = want[[r + at for r in here]]
+            err = np.abs(got - ref).max(axis=1)
+            assert err.max() <= TOL["bfloat16"] * np.abs(want).max(), (cuts, at, err)
+            at += n
+        runner.release("x")
+
+
 # ---------------------------------------------- keys at the window's edges and at the kept ones' ---
 def _needle_model(tmp_path, window, keep_first, heads=2, dim=16, vdim=16):
     """One layer of two-map attention whose keys are its queries (the same matrix and norm weights, as many key heads as
