@@ -230,7 +230,7 @@ class CpuOps:
         w = w / (w.sum(-1, keepdim=True) + 1e-20) * scale if normalize else w * scale
         return ids.to(torch.int32), w, (torch.sigmoid(z[:, experts]) if has_shared else None)
 
-    def apply_experts(self, x, ids, weights, w_gate_up, w_down, packed, shared, shared_gate):
+    def apply_experts(self, x, ids, weights, w_gate_up, w_down, packed, shared, shared_gate, limit=0.0, slope=1.0):
         T, n = x.shape
         E = w_gate_up.shape[0]
         ff = w_gate_up.shape[1] // 2
@@ -243,7 +243,7 @@ class CpuOps:
                     out[t] += weights[t, j] * xf[t]
                     continue
                 gu = w_gate_up[e].to(torch.float32) @ xf[t]
-                a = (gu[:ff] / (1 + torch.exp(-gu[:ff])) * gu[ff:]).to(x.dtype).to(torch.float32)
+                a = self._gated(gu[:ff], gu[ff:], limit, slope).to(x.dtype).to(torch.float32)
                 out[t] += weights[t, j] * (w_down[e].to(torch.float32) @ a)
         if shared is not None:
             out = out + (shared.to(torch.float32) if shared_gate is None else shared_gate[:, None] * shared.to(torch.float32))
@@ -304,7 +304,7 @@ class CpuOps:
         return out.reshape(T, heads * vdim).to(proj.dtype)
 
     def latent_attention(self, proj, step, cache, heads, dim, rot, rank, vdim, norm_weight, norm_eps, rotary, scale,
-                         w_qk, w_v):
+                         w_qk, w_v, sinks=None):
         T = step.num_rows
         x = proj.to(torch.float32)
         cos, sin, rd = rotary
@@ -332,7 +332,10 @@ class CpuOps:
             pg = tables[int(seq[r]), idx // page].long()
             assert (pg >= 0).all(), "a row reads a page that is not held"
             kk = kc[pg, idx % page].to(torch.float32)               # [n, rank + rot]
-            w = torch.softmax((qk[r] @ kk.t()) * scale, dim=-1)     # [heads, n]
+            sc = (qk[r] @ kk.t()) * scale                           # [heads, n]
+            if sinks is not None:
+                sc = torch.cat([sc, sinks[:, None]], dim=-1)
+            w = torch.softmax(sc, dim=-1)[:, :len(idx)]
             o[r] = w @ kk[:, :rank]
         o = o.to(proj.dtype).to(torch.float32)
         return torch.einsum("thn,hen->the", o, w_v.to(torch.float32)).reshape(T, heads * vdim).to(proj.dtype)
@@ -360,10 +363,93 @@ class CpuOps:
     def linear_swiglu(self, x, m):
         return self.swiglu(self.linear(x, m))
 
-    def swiglu(self, gu):
+    @staticmethod
+    def _gated(g, u, limit, slope):
+        if limit <= 0:
+            return g / (1 + torch.exp(-g)) * u
+        g, u = torch.clamp(g, max=limit), torch.clamp(u, min=-limit, max=limit)
+        return g / (1 + torch.exp(-slope * g)) * (u + 1)
+
+    def swiglu(self, gu, limit=0.0, slope=1.0):
         inter = gu.shape[1] // 2
         g, u = gu[:, :inter].to(torch.float32), gu[:, inter:].to(torch.float32)
-        return (g / (1 + torch.exp(-g)) * u).to(gu.dtype)
+        return self._gated(g, u, limit, slope).to(gu.dtype)
+
+    # ---- attention with biases and a sink whose values may be its keys; lightning attention ----
+    def sink_attention(self, proj, step, cache, heads, kv_heads, head_dim, bias, rotary, scale, sinks, window,
+                       values_are_keys):
+        T = step.num_rows
+        qd, kd = heads * head_dim, kv_heads * head_dim
+        x = proj.to(torch.float32)
+        if bias is not None:
+            x = x + bias
+        q = x[:, :qd].reshape(T, heads, head_dim)
+        k = x[:, qd:qd + kd].reshape(T, kv_heads, head_dim)
+        v = k if values_are_keys else x[:, qd + kd:].reshape(T, kv_heads, head_dim)
+        pos, seq = step.positions.long(), step.seq_of_row.long()
+        if rotary is not None:
+            cos, sin, rd = rotary
+            half = rd // 2
+            c, s_ = cos[pos][:, None, :], sin[pos][:, None, :]
+
+            def rot(t):
+                a, b, rest = t[..., :half], t[..., half:rd], t[..., rd:]
+                return torch.cat([a * c - b * s_, b * c + a * s_, rest], dim=-1)
+            q, k = rot(q), rot(k)
+        page, tables = cache.group.page_size, cache.group.tables
+        pages = tables[seq, pos // page].long()
+        assert (pages >= 0).all(), "a row writes to a page that is not held"
+        kc, vc = cache.record("k"), cache.record("v")
+        kc[pages, :, pos % page] = k.to(kc.dtype)
+        vc[pages, :, :, pos % page] = v.to(vc.dtype)
+        q = q.to(proj.dtype).to(torch.float32)
+        out = torch.zeros(T, heads, head_dim)
+        mul = heads // kv_heads
+        for r in range(T):
+            idx = self._seen(int(pos[r]), window, 0)
+            pg = tables[int(seq[r]), idx // page].long()
+            assert (pg >= 0).all(), "a row reads a page that is not held"
+            kk = kc[pg, :, idx % page].to(torch.float32)            # [n, kv, d]
+            vv = vc[pg, :, :, idx % page].to(torch.float32)
+            for h in range(heads):
+                sc = (kk[:, h // mul] @ q[r, h]) * scale
+                if sinks is not None:
+                    sc = torch.cat([sc, sinks[h:h + 1]])
+                w = torch.softmax(sc, dim=0)[:len(idx)]
+                out[r, h] = w @ vv[:, h // mul]
+        return out.reshape(T, qd).to(proj.dtype)
+
+    def add_bias(self, y, bias):
+        return (y.to(torch.float32) + bias).to(y.dtype)
+
+    def check_lightning_sizes(self, heads, dk, dv):
+        pass
+
+    def lightning_state_shape(self, heads, dk, dv):
+        return (heads, dv, dk)
+
+    def lightning_attention(self, proj, decay, state, step, heads, dk, dv):
+        T = step.num_rows
+        x = proj.to(torch.float32)
+        x = x / (1 + torch.exp(-x))
+        q = x[:, :heads * dk].reshape(T, heads, dk)
+        k = x[:, heads * dk:2 * heads * dk].reshape(T, heads, dk)
+        v = x[:, 2 * heads * dk:2 * heads * dk + heads * dv].reshape(T, heads, dv)
+        out = torch.zeros(T, heads, dv)
+        for i in range(step.num_seqs):
+            r0, r1 = step.h_row_start[i], step.h_row_start[i + 1]
+            slot = step.h_slots[i]
+            S = state[slot].clone() if step.h_seq_start[i] > 0 else torch.zeros(heads, dv, dk)      # [H, dv, dk]
+            for t in range(r0, r1):
+                S = decay[:, None, None] * S + v[t][:, :, None] * k[t][:, None, :]
+                out[t] = torch.einsum("hvk,hk->hv", S, q[t])
+            state[slot] = S
+        return out.reshape(T, heads * dv)
+
+    def lightning_norm(self, o, proj, gate_at, weight, eps, out_dtype):
+        n = o.shape[1]
+        g = proj[:, gate_at:gate_at + n].to(torch.float32)
+        return (o * torch.rsqrt((o * o).mean(-1, keepdim=True) + eps) * weight * torch.sigmoid(g)).to(out_dtype)
 
     def qkv_to_cache(self, qkv, step, cache, heads, kv_heads, head_dim, q_norm, k_norm, rotary):
         T = step.num_rows

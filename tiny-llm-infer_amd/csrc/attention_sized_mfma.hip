@@ -53,12 +53,22 @@ static inline size_t asm_lds_bytes(int DK, int DV) {
 // EXACT: the sizes are NKM and NVM themselves (nk, nv are not read), so that the loops over a head's sixteens have
 // no conditions left and the compiler orders the LDS reads of one sixteen ahead of the matrix instruction of another;
 // with conditions every sixteen is a block of its own that waits for its own reads.
+// A sink: a learned logit a (head, map) that stands in the softmax's denominator with no key and no value.  With the
+// running maximum m and sum l (of exp(s - m)) over a row's keys, the row's output is acc / (l + exp(sink - m)); the
+// factor that the accumulators are multiplied with, written so that neither exponential overflows.
+__device__ __forceinline__ float asm_sink_factor(float sink, float m, float l) {
+    const float top = fmaxf(m, sink);
+    const float keys = (m == -INFINITY) ? 0.f : __expf(m - top);
+    return keys / (l * keys + __expf(sink - top));
+}
+
 template <int NKM, int NVM, bool VKEY, typename TO, bool EXACT>
 __global__ __launch_bounds__(64 * ASM_WAVES) void attention_sized_mfma_kernel(
     const bf16_t* __restrict__ q, TO* __restrict__ out, const bf16_t* __restrict__ k_cache,
     const bf16_t* __restrict__ v_cache, const int* __restrict__ row_start, const int* __restrict__ seq_start,
     int num_seqs, const int* __restrict__ tables, int table_width, int page_size, int num_pages, int heads,
-    int kv_heads, int maps, int nk_arg, int nv_arg, float scale, int window, int keep_first, int grouped, int col_groups) {
+    int kv_heads, int maps, int nk_arg, int nv_arg, float scale, int window, int keep_first, int grouped, int col_groups,
+    const float* __restrict__ sinks) {
     const int nk = EXACT ? NKM : nk_arg, nv = EXACT ? NVM : nv_arg;
     const int DK = nk * 16, DV = nv * 16, LD = DK + ASM_PAD;
     const int pieces = 2 * nk;                                          // 16-byte pieces of one key
@@ -283,7 +293,8 @@ __global__ __launch_bounds__(64 * ASM_WAVES) void attention_sized_mfma_kernel(
         lt += theirs[16 + col] * fw[w];
     }
     if (col >= live_cols) return;
-    const float inv = lt > 0.f ? 1.0f / lt : 0.f;
+    float inv = lt > 0.f ? 1.0f / lt : 0.f;
+    if (sinks) inv = asm_sink_factor(sinks[unit], mt, lt);
     int out_unit = unit, out_row = row0 + my;
     TO* o_row = out + ((size_t)out_row * units + out_unit) * DV;
 #pragma unroll
@@ -328,7 +339,8 @@ __global__ __launch_bounds__(64 * WAVES) void attention_sized_shared_kernel(
     const bf16_t* __restrict__ q, TO* __restrict__ out, const bf16_t* __restrict__ k_cache,
     const bf16_t* __restrict__ v_cache, const int* __restrict__ row_start, const int* __restrict__ seq_start,
     int num_seqs, const int* __restrict__ tables, int table_width, int page_size, int num_pages, int heads,
-    int kv_heads, int maps, int nk_arg, int nv_arg, float scale, int window, int keep_first, int grouped) {
+    int kv_heads, int maps, int nk_arg, int nv_arg, float scale, int window, int keep_first, int grouped,
+    const float* __restrict__ sinks) {
     const int nk = EXACT ? NKM : nk_arg, nv = EXACT ? NVM : nv_arg;
     const int DK = nk * 16, DV = nv * 16, LD = DK + ASM_PAD;
     const int pieces = 2 * nk;                                          // 16-byte pieces of one key
@@ -527,7 +539,8 @@ __global__ __launch_bounds__(64 * WAVES) void attention_sized_shared_kernel(
         __syncthreads();                                // the next tile is written; this one is read by all
     }
     if (!stores || col >= live) return;
-    const float inv = l > 0.f ? 1.0f / l : 0.f;
+    float inv = l > 0.f ? 1.0f / l : 0.f;
+    if (sinks) inv = asm_sink_factor(sinks[unit], m, l);
     TO* o_row = out + ((size_t)row * units + unit) * DV;
 #pragma unroll
     for (int j = 0; j < NVM; ++j)
@@ -545,11 +558,13 @@ extern "C" int tli_attention_sized_mfma_takes(int key_dim, int value_dim, int pa
 // q [rows, heads * maps, key_dim]; out [rows, heads * maps, value_dim] (float32 with out_f32, else bfloat16);
 // k_cache [pages][kv_heads * maps][slot][key_dim]; v_cache [pages][kv_heads][value_dim][slot] or null;
 // tiles: an upper bound of the sum over the sequences of ceil(rows / 16) (of the rows, with `grouped`);
-// grouped: a tile is one row and its columns are the query heads of one key head, 16 at a time
+// grouped: a tile is one row and its columns are the query heads of one key head, 16 at a time;
+// sinks: float32 [heads * maps] or null
 extern "C" int tli_attention_sized_mfma_bf16(
     const void* q, void* out, const void* k_cache, const void* v_cache, const int* row_start, const int* seq_start,
     int num_seqs, int tiles, const int* tables, int table_width, int page_size, int num_pages, int heads, int kv_heads,
-    int maps, int key_dim, int value_dim, float scale, int window, int keep_first, int grouped, int out_f32, void* stream) {
+    int maps, int key_dim, int value_dim, float scale, int window, int keep_first, int grouped, int out_f32,
+    const float* sinks, void* stream) {
     if (num_seqs <= 0 || tiles <= 0) return 0;
     if (!tli_attention_sized_mfma_takes(key_dim, value_dim, page_size, v_cache != nullptr))
         return tli_fail("attention: the matrix-core kernel does not take keys of %d and values of %d in pages of %d", key_dim,
@@ -591,7 +606,7 @@ extern "C" int tli_attention_sized_mfma_bf16(
         }                                                                                                                  \
         kernel<<<sgrid, 64 * WAVES, sbytes, s>>>((const bf16_t*)q, (TO*)out, (const bf16_t*)k_cache, (const bf16_t*)v_cache,      \
                                           row_start, seq_start, num_seqs, tables, table_width, page_size, num_pages,      \
-                                          heads, kv_heads, maps, nk, nv, scale, window, keep_first, grouped);             \
+                                          heads, kv_heads, maps, nk, nv, scale, window, keep_first, grouped, sinks);      \
     }
 #define AST_SIZES(VKEY, TO)                                                   \
     if (nk <= 8 && nv <= 8) AST_ONE(8, 8, VKEY, TO, false, 4)                 \
@@ -631,7 +646,7 @@ extern "C" int tli_attention_sized_mfma_bf16(
         kernel<<<grid, 64 * ASM_WAVES, bytes, s>>>((const bf16_t*)q, (TO*)out, (const bf16_t*)k_cache,                      \
                                                    (const bf16_t*)v_cache, row_start, seq_start, num_seqs, tables,         \
                                                    table_width, page_size, num_pages, heads, kv_heads, maps, nk, nv,       \
-                                                   scale, window, keep_first, grouped, col_groups);                        \
+                                                   scale, window, keep_first, grouped, col_groups, sinks);                 \
     }
 #define ASM_SIZES(VKEY, TO)                                                   \
     if (nk <= 8 && nv <= 8) ASM_ONE(8, 8, VKEY, TO, false)                    \

@@ -7,6 +7,8 @@
 // cache of their own ([page][kv head][value_dim][slot]) or, without one, are the first value_dim elements
 // of the key itself (keys that carry the vector their values are made from).
 //
+// With `sinks` (float32, one a (head, map)) the softmax's denominator also holds exp(sink): a logit without key or value.
+//
 // Row at position p sees key t <= p if p - t < window or t < keep_first (window 0: every t <= p).  The seen
 // keys are walked in one fixed order (the kept first ones, then the window's), 256 at a time with a running
 // maximum and sum; the order of additions depends on (p, window, keep_first) alone, never on the batch.
@@ -20,7 +22,7 @@ __global__ __launch_bounds__(AS_THREADS) void attention_sized_plain_kernel(
     const T* __restrict__ q, TO* __restrict__ out, const T* __restrict__ k_cache, const T* __restrict__ v_cache,
     const int* __restrict__ positions, const int* __restrict__ seq_of_row, const int* __restrict__ tables,
     int table_width, int page_size, int num_pages, int heads, int kv_heads, int maps, int key_dim, int value_dim,
-    float scale, int window, int keep_first) {
+    float scale, int window, int keep_first, const float* __restrict__ sinks) {
     __shared__ float q_s[AS_MAX_DIM];
     __shared__ float p_s[AS_THREADS];
     __shared__ float red[16];
@@ -88,7 +90,12 @@ __global__ __launch_bounds__(AS_THREADS) void attention_sized_plain_kernel(
         __syncthreads();
     }
     TO* o_row = out + ((size_t)row * heads * maps + unit) * value_dim;
-    const float inv = (l > 0.f) ? 1.0f / l : 0.f;
+    float inv = (l > 0.f) ? 1.0f / l : 0.f;
+    if (sinks) {                                                        // the denominator also holds exp(sink)
+        const float top = fmaxf(m, sinks[unit]);
+        const float keys = (m == -INFINITY) ? 0.f : expf(m - top);
+        inv = keys / (l * keys + expf(sinks[unit] - top));
+    }
 #pragma unroll
     for (int part = 0; part < AS_MAX_DIM / AS_THREADS; ++part) {
         const int d = tid + part * AS_THREADS;
@@ -101,7 +108,8 @@ __global__ __launch_bounds__(AS_THREADS) void attention_sized_plain_kernel(
 extern "C" int tli_attention_sized_plain(
     const void* q, void* out, const void* k_cache, const void* v_cache, const int* positions, const int* seq_of_row,
     const int* tables, int table_width, int page_size, int num_pages, int rows, int heads, int kv_heads, int maps,
-    int key_dim, int value_dim, float scale, int window, int keep_first, int dtype, int out_f32, void* stream) {
+    int key_dim, int value_dim, float scale, int window, int keep_first, int dtype, int out_f32, const float* sinks,
+    void* stream) {
     if (rows <= 0) return 0;
     if (key_dim <= 0 || key_dim > AS_MAX_DIM || value_dim <= 0 || value_dim > AS_MAX_DIM)
         return tli_fail("attention: heads of %d and %d elements are outside 1..%d", key_dim, value_dim, AS_MAX_DIM);
@@ -113,7 +121,7 @@ extern "C" int tli_attention_sized_plain(
     if (window < 0 || keep_first < 0) return tli_fail("attention: bad window %d with %d kept", window, keep_first);
     hipStream_t s = (hipStream_t)stream;
     const dim3 grid(rows, heads * maps);
-#define AS_ARGS positions, seq_of_row, tables, table_width, page_size, num_pages, heads, kv_heads, maps, key_dim, value_dim, scale, window, keep_first
+#define AS_ARGS positions, seq_of_row, tables, table_width, page_size, num_pages, heads, kv_heads, maps, key_dim, value_dim, scale, window, keep_first, sinks
     if (dtype == TLI_F32)
         attention_sized_plain_kernel<float, float><<<grid, AS_THREADS, 0, s>>>((const float*)q, (float*)out, (const float*)k_cache,
                                                                                (const float*)v_cache, AS_ARGS);

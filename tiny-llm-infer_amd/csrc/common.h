@@ -75,6 +75,15 @@ __device__ __forceinline__ void store4(bf16_t* dst, const float (&v)[4], int lef
         if (i < left) dst[i] = f32_to_bf16(v[i]);
 }
 
+// What a gated feed-forward makes of a gate sum g and an up sum u.  limit <= 0: silu(g) * u.  limit > 0, the limited
+// form: g <- min(g, limit), u <- clamp(u, -limit, limit), then g * sigmoid(slope * g) * (u + 1).
+__device__ __forceinline__ float gated_unit(float g, float u, float limit, float slope) {
+    if (limit <= 0.f) return g / (1.0f + expf(-g)) * u;
+    g = fminf(g, limit);
+    u = fminf(fmaxf(u, -limit), limit);
+    return g / (1.0f + expf(-slope * g)) * (u + 1.0f);
+}
+
 // Makes LDS writes of this wavefront's lanes visible to its other lanes.
 __device__ __forceinline__ void wave_lds_sync() {
     __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");

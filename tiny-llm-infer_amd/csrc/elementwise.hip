@@ -194,14 +194,15 @@ static void launch_add_rmsnorm(float* resid, const void* delta, int parts, const
 }
 
 template <typename T>
-__global__ void swiglu_kernel(const T* __restrict__ gu, T* __restrict__ out, int inter, size_t total) {
+__global__ void swiglu_kernel(const T* __restrict__ gu, T* __restrict__ out, int inter, size_t total, float limit,
+                              float slope) {
     size_t idx = (size_t)blockIdx.x * blockDim.x + threadIdx.x;
     if (idx >= total) return;
     const size_t row = idx / inter;
     const int col = (int)(idx - row * inter);
     const float g = to_f32(gu[row * 2 * inter + col]);
     const float u = to_f32(gu[row * 2 * inter + inter + col]);
-    from_f32(out + idx, g / (1.0f + expf(-g)) * u);
+    from_f32(out + idx, gated_unit(g, u, limit, slope));
 }
 
 // token_ids[r] = src[from[r]] where from[r] >= 0: the tokens a step sampled become the
@@ -256,7 +257,7 @@ extern "C" int tli_add_rmsnorm(float* resid, const void* delta, const float* wei
 
 // 8 outputs a thread, 16-byte loads: inter % 8 == 0
 __global__ void swiglu_vec_kernel(const bf16_t* __restrict__ gu, bf16_t* __restrict__ out, int inter,
-                                  size_t groups) {
+                                  size_t groups, float limit, float slope) {
     const size_t idx = (size_t)blockIdx.x * blockDim.x + threadIdx.x;
     if (idx >= groups) return;
     const int per_row = inter / 8;
@@ -270,25 +271,26 @@ __global__ void swiglu_vec_kernel(const bf16_t* __restrict__ gu, bf16_t* __restr
     for (int i = 0; i < 4; ++i) {
         const float g0 = bf16_to_f32((bf16_t)(gw[i] & 0xffffu)), g1 = bf16_to_f32((bf16_t)(gw[i] >> 16));
         const float u0 = bf16_to_f32((bf16_t)(uw[i] & 0xffffu)), u1 = bf16_to_f32((bf16_t)(uw[i] >> 16));
-        const float a0 = g0 / (1.0f + expf(-g0)) * u0, a1 = g1 / (1.0f + expf(-g1)) * u1;
+        const float a0 = gated_unit(g0, u0, limit, slope), a1 = gated_unit(g1, u1, limit, slope);
         ow[i] = (uint32_t)f32_to_bf16(a0) | ((uint32_t)f32_to_bf16(a1) << 16);
     }
     *reinterpret_cast<uint4*>(out + row * inter + col) = make_uint4(ow[0], ow[1], ow[2], ow[3]);
 }
 
-extern "C" int tli_swiglu(const void* gu, void* out, int rows, int inter, int dtype, void* stream) {
+// limit, slope: the activation (common.h's gated_unit; limit 0: silu(gate) * up)
+extern "C" int tli_swiglu(const void* gu, void* out, int rows, int inter, int dtype, float limit, float slope, void* stream) {
     if (rows <= 0) return 0;
     if (inter <= 0) return tli_fail("swiglu: bad size %d", inter);
     hipStream_t s = (hipStream_t)stream;
     const size_t total = (size_t)rows * inter;
     const unsigned blocks = (unsigned)((total + 255) / 256);
     if (dtype == TLI_F32)
-        swiglu_kernel<float><<<blocks, 256, 0, s>>>((const float*)gu, (float*)out, inter, total);
+        swiglu_kernel<float><<<blocks, 256, 0, s>>>((const float*)gu, (float*)out, inter, total, limit, slope);
     else if (dtype == TLI_BF16 && inter % 8 == 0) {
         const size_t groups = total / 8;
-        swiglu_vec_kernel<<<(unsigned)((groups + 255) / 256), 256, 0, s>>>((const bf16_t*)gu, (bf16_t*)out, inter, groups);
+        swiglu_vec_kernel<<<(unsigned)((groups + 255) / 256), 256, 0, s>>>((const bf16_t*)gu, (bf16_t*)out, inter, groups, limit, slope);
     } else if (dtype == TLI_BF16)
-        swiglu_kernel<bf16_t><<<blocks, 256, 0, s>>>((const bf16_t*)gu, (bf16_t*)out, inter, total);
+        swiglu_kernel<bf16_t><<<blocks, 256, 0, s>>>((const bf16_t*)gu, (bf16_t*)out, inter, total, limit, slope);
     else
         return tli_fail("swiglu: unknown dtype %d", dtype);
     return tli_check_launch("swiglu");

@@ -1,0 +1,187 @@
+// Lightning attention: a matrix of state a head that decays by a constant a token.
+//
+// For the rows of one sequence and head h (key size dk, value size dv, decay c_h from the caller):
+//   q_t = silu(proj q),  k_t = silu(proj k),  v_t = silu(proj v)          (float32 from the projections' storage type)
+//   S_t = c_h S_(t-1) + k_t v_t^T        S [dk, dv], float32, zero before position 0
+//   o_t = S_t^T q_t                      float32
+// The state of a sequence lives in its slot between steps, transposed ([head][dv][dk]: the dk elements of a column
+// lie together), so that a wave reads and writes it in runs.  A sequence that starts at position 0 does not read its
+// slot: slots are never cleared when they change hands.
+//
+// Columns of S are independent.  A workgroup takes LT_COLS columns of one head of one sequence and walks the
+// sequence's rows in order; a column belongs to the 16 lanes of a DPP row, lane s holding elements s R .. s R + R - 1
+// of it in registers (R = dk / 16 rounded up to a power of two; elements from dk on stay zero).  A row costs R
+// multiply-adds for the state, R for the output and four DPP moves.  The rows come through LDS in chunks that the
+// whole workgroup fetches (with the silu) into registers while the chunk before is walked.
+//
+// lightning_norm: y = o / sqrt(mean(o^2) + eps) * w * sigmoid(gate) over all heads of a row together.
+#include "common.h"
+
+#define LT_THREADS 256
+#define LT_COLS 16
+#define LT_MAX_DK 256
+
+__device__ __forceinline__ float lt_silu(float z) { return z / (1.0f + expf(-z)); }
+
+// sum over the 16 lanes of a DPP row; every lane gets it
+__device__ __forceinline__ float lt_sum16(float v) {
+    v += __int_as_float(__builtin_amdgcn_update_dpp(0, __float_as_int(v), 0xB1, 0xF, 0xF, true));     // neighbours
+    v += __int_as_float(__builtin_amdgcn_update_dpp(0, __float_as_int(v), 0x4E, 0xF, 0xF, true));     // pairs of a quad
+    v += __int_as_float(__builtin_amdgcn_update_dpp(0, __float_as_int(v), 0x141, 0xF, 0xF, true));    // halves mirrored
+    v += __int_as_float(__builtin_amdgcn_update_dpp(0, __float_as_int(v), 0x140, 0xF, 0xF, true));    // row mirrored
+    return v;
+}
+
+template <typename T, int R, int CH>
+__global__ __launch_bounds__(LT_THREADS) void lightning_recurrence_kernel(
+    const T* __restrict__ proj, int ld, const float* __restrict__ decay, float* __restrict__ state,
+    float* __restrict__ out, const int* __restrict__ row_start, const int* __restrict__ seq_start,
+    const int* __restrict__ slots, int H, int dk, int dv) {
+    constexpr int DKP = 16 * R;
+    constexpr int W = 2 * DKP + LT_COLS;                 // floats of a staged row: q, k, the workgroup's values
+    constexpr int PF = CH * W / LT_THREADS;
+    static_assert(PF * LT_THREADS == CH * W, "a chunk is shared out evenly");
+    __shared__ __align__(16) float rows_s[CH * W];
+    const int seq = blockIdx.z, h = blockIdx.y, j0 = blockIdx.x * LT_COLS;
+    const int tid = threadIdx.x, lane = tid % TLI_WAVE, wave = tid / TLI_WAVE;
+    const int sub = lane % 16, jl = wave * 4 + lane / 16;
+    const int j = j0 + jl;
+    const int r0 = row_start[seq], n = row_start[seq + 1] - r0;
+    if (n <= 0) return;
+    const float lam = decay[h];
+    float* col = state + (((size_t)slots[seq] * H + h) * dv + (j < dv ? j : 0)) * dk;
+    const bool whole = dk == DKP && R % 4 == 0;          // the lane's elements as 16-byte pieces
+    float S[R];
+#pragma unroll
+    for (int r = 0; r < R; ++r) S[r] = 0.f;
+    if (seq_start[seq] != 0 && j < dv) {
+        if (whole) {
+#pragma unroll
+            for (int r = 0; r < R / 4 * 4; r += 4) {
+                const float4 v = *reinterpret_cast<const float4*>(col + sub * R + r);
+                S[r] = v.x, S[r + 1] = v.y, S[r + 2] = v.z, S[r + 3] = v.w;
+            }
+        } else {
+#pragma unroll
+            for (int r = 0; r < R; ++r)
+                if (sub * R + r < dk) S[r] = col[sub * R + r];
+        }
+    }
+    const size_t q_at = (size_t)h * dk, k_at = (size_t)H * dk + (size_t)h * dk, v_at = (size_t)2 * H * dk + (size_t)h * dv;
+    float pf[PF];
+    auto fetch = [&](int first) {
+#pragma unroll
+        for (int u = 0; u < PF; ++u) {
+            const int e = tid + u * LT_THREADS;
+            const int t = first + e / W, cc = e % W;
+            float val = 0.f;
+            if (t < n) {
+                const T* src = proj + (size_t)(r0 + t) * ld;
+                if (cc < DKP) {
+                    if (cc < dk) val = lt_silu(to_f32(src[q_at + cc]));
+                } else if (cc < 2 * DKP) {
+                    if (cc - DKP < dk) val = lt_silu(to_f32(src[k_at + cc - DKP]));
+                } else if (j0 + cc - 2 * DKP < dv) {
+                    val = lt_silu(to_f32(src[v_at + j0 + cc - 2 * DKP]));
+                }
+            }
+            pf[u] = val;
+        }
+    };
+    fetch(0);
+    float* o_col = out + (size_t)r0 * H * dv + (size_t)h * dv + j;
+    for (int t0 = 0; t0 < n; t0 += CH) {
+        __syncthreads();                                 // the chunk before has been walked by every wave
+#pragma unroll
+        for (int u = 0; u < PF; ++u) rows_s[tid + u * LT_THREADS] = pf[u];
+        __syncthreads();
+        if (t0 + CH < n) fetch(t0 + CH);
+        const int cnt = min(CH, n - t0);
+        for (int t = 0; t < cnt; ++t) {
+            const float* row = rows_s + t * W;
+            const float v = row[2 * DKP + jl];
+            float acc = 0.f;
+#pragma unroll
+            for (int r = 0; r < R; ++r) {
+                S[r] = fmaf(lam, S[r], row[DKP + sub * R + r] * v);
+                acc = fmaf(S[r], row[sub * R + r], acc);
+            }
+            acc = lt_sum16(acc);
+            if (sub == 0 && j < dv) o_col[(size_t)(t0 + t) * H * dv] = acc;
+        }
+    }
+    if (j >= dv) return;
+    if (whole) {
+#pragma unroll
+        for (int r = 0; r < R / 4 * 4; r += 4)
+            *reinterpret_cast<float4*>(col + sub * R + r) = make_float4(S[r], S[r + 1], S[r + 2], S[r + 3]);
+    } else {
+#pragma unroll
+        for (int r = 0; r < R; ++r)
+            if (sub * R + r < dk) col[sub * R + r] = S[r];
+    }
+}
+
+// proj: [T, ld] raw projections, q (H dk), k (H dk), v (H dv) first; decay: float32 [H]; state: float32
+// [slots, H, dv, dk]; out: float32 [T, H dv]; row_start [seqs + 1], seq_start, slots [seqs]
+extern "C" int tli_lightning_recurrence(const void* proj, int ld, const float* decay, float* state, float* out,
+                                        const int* row_start, const int* seq_start, const int* slots, int seqs, int H,
+                                        int dk, int dv, int dtype, void* stream) {
+    if (seqs <= 0) return 0;
+    if (H <= 0 || dk <= 0 || dv <= 0 || dk > LT_MAX_DK)
+        return tli_fail("lightning: bad sizes (heads %d, keys of %d (at most %d), values of %d)", H, dk, LT_MAX_DK, dv);
+    if (ld < 2 * H * dk + H * dv) return tli_fail("lightning: rows of %d hold fewer than q, k and v", ld);
+    if (H > 65535 || seqs > 65535) return tli_fail("lightning: too many heads or sequences for one launch");
+    const dim3 grid((dv + LT_COLS - 1) / LT_COLS, H, seqs);
+    hipStream_t s = (hipStream_t)stream;
+    const int need = (dk + 15) / 16;
+#define LT_LAUNCH(T, R, CH)                                                                                             \
+    hipLaunchKernelGGL((lightning_recurrence_kernel<T, R, CH>), grid, dim3(LT_THREADS), 0, s, (const T*)proj, ld, decay, \
+                       state, out, row_start, seq_start, slots, H, dk, dv)
+#define LT_SIZES(T)                      \
+    if (need <= 1) LT_LAUNCH(T, 1, 32);  \
+    else if (need <= 2) LT_LAUNCH(T, 2, 32); \
+    else if (need <= 4) LT_LAUNCH(T, 4, 32); \
+    else if (need <= 8) LT_LAUNCH(T, 8, 32); \
+    else LT_LAUNCH(T, 16, 16)
+    if (dtype == TLI_F32) { LT_SIZES(float); }
+    else if (dtype == TLI_BF16) { LT_SIZES(bf16_t); }
+    else return tli_fail("lightning: unknown dtype %d", dtype);
+#undef LT_SIZES
+#undef LT_LAUNCH
+    return tli_check_launch("lightning_recurrence");
+}
+
+// one workgroup a row
+template <typename T>
+__global__ void lightning_norm_kernel(const float* __restrict__ o, const T* __restrict__ gate, int gate_ld,
+                                      const float* __restrict__ weight, T* __restrict__ out, int n, float eps) {
+    __shared__ float red[16];
+    const size_t row = blockIdx.x;
+    const float* x = o + row * n;
+    const T* g = gate + row * gate_ld;
+    float ss = 0.f;
+    for (int i = threadIdx.x; i < n; i += blockDim.x) ss += x[i] * x[i];
+    ss = block_sum(ss, red);
+    const float scale = 1.0f / sqrtf(ss / (float)n + eps);
+    for (int i = threadIdx.x; i < n; i += blockDim.x)
+        from_f32(out + row * n + i, x[i] * scale * weight[i] / (1.0f + expf(-to_f32(g[i]))));
+}
+
+// o: float32 [T, n]; gate: [T, gate_ld] (its first n columns); weight: float32 [n]; out: [T, n]
+extern "C" int tli_lightning_norm(const float* o, const void* gate, int gate_ld, const float* weight, void* out, int T,
+                                  int n, float eps, int dtype, void* stream) {
+    if (T <= 0) return 0;
+    if (n <= 0 || gate_ld < n) return tli_fail("lightning_norm: bad sizes");
+    hipStream_t s = (hipStream_t)stream;
+    const int threads = n >= 2048 ? 512 : 256;
+    if (dtype == TLI_F32)
+        hipLaunchKernelGGL((lightning_norm_kernel<float>), dim3(T), dim3(threads), 0, s, o, (const float*)gate, gate_ld, weight,
+                           (float*)out, n, eps);
+    else if (dtype == TLI_BF16)
+        hipLaunchKernelGGL((lightning_norm_kernel<bf16_t>), dim3(T), dim3(threads), 0, s, o, (const bf16_t*)gate, gate_ld,
+                           weight, (bf16_t*)out, n, eps);
+    else
+        return tli_fail("lightning_norm: unknown dtype %d", dtype);
+    return tli_check_launch("lightning_norm");
+}

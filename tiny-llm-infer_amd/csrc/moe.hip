@@ -9,7 +9,8 @@
 //          or s_j * scale without that division.  One more logit behind the E, if present, is the gate of
 //          a shared expert: sigmoid of it.  Ids from `experts` on (see the kernels below) are experts that
 //          hand their input on: they have no matrices.
-// hidden:  for the pair (row, chosen expert e): a_f = silu(x . Wg_e[f]) * (x . Wu_e[f])
+// hidden:  for the pair (row, chosen expert e): a_f = silu(x . Wg_e[f]) * (x . Wu_e[f]), or the limited form of
+//          common.h's gated_unit (limit > 0)
 // down:    y_c = sum_j weight_j (a_j . Wd_e(j)[c])  (+ shared gate * shared_c), summed in the order of
 //          the choice, so that a row's result does not depend on what else is in the step.
 //
@@ -88,12 +89,10 @@ __global__ void moe_route_kernel(const float* __restrict__ z, long long z_row, l
     }
 }
 
-__device__ __forceinline__ float moe_silu(float z) { return z / (1.0f + expf(-z)); }
-
 // one workgroup a pair; a wave takes every (waves)th hidden unit, its lanes share out k
 template <typename T>
 __global__ void moe_hidden_kernel(const T* __restrict__ x, const int* __restrict__ ids, const T* __restrict__ w_gu,
-                                  T* __restrict__ hid, int top, int D, int ff, int E) {
+                                  T* __restrict__ hid, int top, int D, int ff, int E, float limit, float slope) {
     extern __shared__ float xs[];                  // the pair's input row
     const int pair = blockIdx.x;
     const int t = pair / top;
@@ -114,7 +113,7 @@ __global__ void moe_hidden_kernel(const T* __restrict__ x, const int* __restrict
         }
         a = wave_sum(a);
         b = wave_sum(b);
-        if (lane == 0) from_f32(hid + (size_t)pair * ff + f, moe_silu(a) * b);
+        if (lane == 0) from_f32(hid + (size_t)pair * ff + f, gated_unit(a, b, limit, slope));
     }
 }
 
@@ -168,10 +167,10 @@ extern "C" int tli_moe_route(const float* z, long long z_row, long long z_col, i
 
 // x [T, D]; ids, weights [T, top]; w_gu [E, 2 ff, D] (an expert's gate rows, then its up rows);
 // w_down [E, D, ff]; hid [T * top, ff] is scratch; shared [T, D] or null (shared_gate null: added as it is); out [T, D];
-// an id outside 0..E-1 is an expert that hands its input on
+// an id outside 0..E-1 is an expert that hands its input on; limit, slope: the activation (gated_unit)
 extern "C" int tli_moe_experts(const void* x, const int* ids, const float* weights, const void* w_gu,
                                const void* w_down, void* hid, const void* shared, const float* shared_gate, void* out,
-                               int T, int top, int D, int ff, int E, int dtype, void* stream) {
+                               int T, int top, int D, int ff, int E, int dtype, float limit, float slope, void* stream) {
     if (T <= 0) return 0;
     if (top <= 0 || D <= 0 || ff <= 0) return tli_fail("moe_experts: bad sizes");
     if ((size_t)D * 4 > 64 * 1024 || (size_t)top * ff * 4 > 64 * 1024)
@@ -182,12 +181,12 @@ extern "C" int tli_moe_experts(const void* x, const int* ids, const float* weigh
     const dim3 dgrid((D + cols - 1) / cols, T);
     if (dtype == TLI_F32) {
         hipLaunchKernelGGL((moe_hidden_kernel<float>), dim3(T * top), dim3(256), (size_t)D * 4, s, (const float*)x, ids,
-                           (const float*)w_gu, (float*)hid, top, D, ff, E);
+                           (const float*)w_gu, (float*)hid, top, D, ff, E, limit, slope);
         hipLaunchKernelGGL((moe_down_kernel<float>), dgrid, dim3(256), (size_t)top * ff * 4, s, (const float*)hid, ids,
                            weights, (const float*)w_down, (const float*)shared, shared_gate, (float*)out, top, D, ff, cols, E, (const float*)x);
     } else if (dtype == TLI_BF16) {
         hipLaunchKernelGGL((moe_hidden_kernel<bf16_t>), dim3(T * top), dim3(256), (size_t)D * 4, s, (const bf16_t*)x, ids,
-                           (const bf16_t*)w_gu, (bf16_t*)hid, top, D, ff, E);
+                           (const bf16_t*)w_gu, (bf16_t*)hid, top, D, ff, E, limit, slope);
         hipLaunchKernelGGL((moe_down_kernel<bf16_t>), dgrid, dim3(256), (size_t)top * ff * 4, s, (const bf16_t*)hid, ids,
                            weights, (const bf16_t*)w_down, (const bf16_t*)shared, shared_gate, (bf16_t*)out, top, D, ff,
                            cols, E, (const bf16_t*)x);

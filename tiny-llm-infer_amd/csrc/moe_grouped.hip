@@ -5,7 +5,8 @@
 //             tiles of RT slots (`order`: slot -> pair or -1, `pos`: pair -> slot, `tile_expert`: tile ->
 //             expert).  How many tiles there are is known on the device only: the products are launched
 //             for the most there can be (pairs / RT + experts) and a workgroup without a tile leaves.
-//   gate/up:  hid[slot, f] = silu(x[row] . Wg_e[f]) * (x[row] . Wu_e[f])          (bfloat16)
+//   gate/up:  hid[slot, f] = silu(x[row] . Wg_e[f]) * (x[row] . Wu_e[f])          (bfloat16; or the limited form of
+//             common.h's gated_unit)
 //   down:     part[slot, c] = hid[slot] . Wd_e[c]                                 (float32)
 //   combine:  y[row] = sum_j weight[row, j] part[pos[row, j]]  (+ shared gate * shared), in the order of
 //             the choice: a row's result does not depend on which other rows share its tiles, because the
@@ -213,8 +214,6 @@ __device__ __forceinline__ void tile_product(const bf16_t* __restrict__ a1, cons
     }
 }
 
-__device__ __forceinline__ float grouped_silu(float z) { return z / (1.0f + expf(-z)); }
-
 // gate and up products with the activation: hid[slot, f] (a tile has 16 RB slots)
 template <int RB, int NB>
 __global__ void __launch_bounds__(256) moe_gate_up_kernel(const bf16_t* __restrict__ x, const int* __restrict__ order,
@@ -222,7 +221,7 @@ __global__ void __launch_bounds__(256) moe_gate_up_kernel(const bf16_t* __restri
                                                            const int* __restrict__ num_tiles,
                                                            const bf16_t* __restrict__ gate_t,
                                                            const bf16_t* __restrict__ up_t, bf16_t* __restrict__ hid,
-                                                           int top, int D, int ff) {
+                                                           int top, int D, int ff, float limit, float slope) {
     __shared__ __attribute__((aligned(16))) bf16_t xt[16 * RB * XT_STRIDE];
     __shared__ long long src_off[16 * RB];
     const int tile = blockIdx.y;
@@ -257,7 +256,7 @@ __global__ void __launch_bounds__(256) moe_gate_up_kernel(const bf16_t* __restri
             if (src_off[b * 16 + r] < 0) continue;
             float h[4];
 #pragma unroll
-            for (int v = 0; v < 4; ++v) h[v] = grouped_silu(ag[i][b][v]) * au[i][b][v];
+            for (int v = 0; v < 4; ++v) h[v] = gated_unit(ag[i][b][v], au[i][b][v], limit, slope);
             store4(hid + (size_t)((tile * RB + b) * 16 + r) * ff + n0, h, ff - n0, ff % 4 == 0);
         }
     }
@@ -341,7 +340,7 @@ extern "C" int tli_moe_grouped_bf16(const void* x, const int* ids, const float* 
                                     const void* up_t, const void* down_t, int* order, int* pos, int* tile_expert,
                                     int* num_tiles, void* hid, float* part, const void* shared,
                                     const float* shared_gate, void* out, int T, int top, int E, int D, int ff, int RT,
-                                    void* stream) {
+                                    float limit, float slope, void* stream) {
     if (T <= 0) return 0;
     if (top <= 0 || E <= 0 || E > SORT_MAX_EXPERTS || D <= 0 || ff <= 0 || D % 8 || ff % 8)
         return tli_fail("moe_grouped: bad sizes (experts %d (at most %d), width %d and hidden units %d in eights)", E,
@@ -357,7 +356,7 @@ extern "C" int tli_moe_grouped_bf16(const void* x, const int* ids, const float* 
 #define TLI_GROUPED(RB, NBG)                                                                                          \
     hipLaunchKernelGGL((moe_gate_up_kernel<RB, NBG>), dim3((ff + 64 * NBG - 1) / (64 * NBG), (unsigned)tiles_max),      \
                        dim3(256), 0, s, (const bf16_t*)x, order, tile_expert, num_tiles, (const bf16_t*)gate_t,        \
-                       (const bf16_t*)up_t, (bf16_t*)hid, top, D, ff);                                                 \
+                       (const bf16_t*)up_t, (bf16_t*)hid, top, D, ff, limit, slope);                                   \
     hipLaunchKernelGGL((moe_down_grouped_kernel<RB, 2>), dim3((D + 127) / 128, (unsigned)tiles_max), dim3(256), 0, s,  \
                        (const bf16_t*)hid, order, tile_expert, num_tiles, (const bf16_t*)down_t, part, D, ff)
     if (RT == 16) { TLI_GROUPED(1, 2); }

@@ -75,7 +75,7 @@ def load_library():
         "tli_embed": [P, P, P, I, I, I, I, P],
         "tli_feed_tokens": [P, P, P, I, I, P],
         "tli_add_rmsnorm": [P, P, P, P, P, I, I, I, F, I, I, P],
-        "tli_swiglu": [P, P, I, I, I, P],
+        "tli_swiglu": [P, P, I, I, I, F, F, P],
         "tli_qkv_to_cache": [P, P, P, P, P, P, P, I, I, I, I, I, I, I, P, F, P, F, P, P, I, I, I, I, I, P],
         "tli_values_to_cache": [P, P, P, P, I, I, P, I, I, I, I, I, I, P],
         "tli_keys_values_to_cache": [P, P, P, P, P, I, I, P, I, I, I, I, I, I, P, F, P, P, I, P],
@@ -110,22 +110,26 @@ def load_library():
         "tli_delta_state_floats": [I, I],
         "tli_gated_rmsnorm": [P, P, I, P, P, I, I, I, F, I, P],
         "tli_moe_route": [P, ctypes.c_longlong, ctypes.c_longlong, P, P, P, I, I, I, I, I, F, I, I, I, I, P, P],
-        "tli_moe_experts": [P, P, P, P, P, P, P, P, P, I, I, I, I, I, I, P],
+        "tli_moe_experts": [P, P, P, P, P, P, P, P, P, I, I, I, I, I, I, F, F, P],
         "tli_norm_add": [P, P, P, P, I, I, F, I, P],
         "tli_residual_rows": [P, P, ctypes.c_longlong, P],
-        "tli_attention_sized_plain": [P, P, P, P, P, P, P, I, I, I, I, I, I, I, I, I, F, I, I, I, I, P],
+        "tli_attention_sized_plain": [P, P, P, P, P, P, P, I, I, I, I, I, I, I, I, I, F, I, I, I, I, P, P],
         "tli_attention_sized_mfma_takes": [I, I, I, I],
         "tli_head_products_mfma_takes": [I, I] + [ctypes.c_longlong] * 4,
         "tli_head_products_mfma_bf16": [P, ctypes.c_longlong, ctypes.c_longlong, P, P, ctypes.c_longlong, ctypes.c_longlong,
                                         I, I, I, I, P],
-        "tli_attention_sized_mfma_bf16": [P, P, P, P, P, P, I, I, P, I, I, I, I, I, I, I, I, F, I, I, I, I, P],
+        "tli_attention_sized_mfma_bf16": [P, P, P, P, P, P, I, I, P, I, I, I, I, I, I, I, I, F, I, I, I, I, P, P],
         "tli_diff_prepare": [P, I, P, P, P, P, P, P, I, I, I, I, I, I, I, I, P, P, F, I, P],
         "tli_diff_combine": [P, P, I, I, P, I, I, I, F, F, F, I, P],
         "tli_latent_prepare": [P, I, P, P, P, P, P, I, I, I, I, I, I, I, I, I, P, F, P, P, I, P],
         "tli_head_products_plain": [P, ctypes.c_longlong, ctypes.c_longlong, P, P, ctypes.c_longlong, ctypes.c_longlong,
                                     I, I, I, I, I, P],
         "tli_moe_grouped_tile": [I, I],
-        "tli_moe_grouped_bf16": [P, P, P, P, P, P, P, P, P, P, P, P, P, P, P, I, I, I, I, I, I, P],
+        "tli_moe_grouped_bf16": [P, P, P, P, P, P, P, P, P, P, P, P, P, P, P, I, I, I, I, I, I, F, F, P],
+        "tli_keyed_prepare": [P, I, P, P, P, P, P, P, P, I, I, I, I, I, I, I, I, P, P, I, I, I, P],
+        "tli_add_bias": [P, P, I, I, I, P],
+        "tli_lightning_recurrence": [P, I, P, P, P, P, P, P, I, I, I, I, I, P],
+        "tli_lightning_norm": [P, P, I, P, P, I, I, F, I, P],
         "tli_sample": [P, I, I, P, P, P, P, P, P],
         "tli_sample_scratch_bytes": [I],
         "tli_random_normal": [P, ctypes.c_longlong, ctypes.c_uint32, ctypes.c_uint32, ctypes.c_uint32, P, F, F, I, P],
@@ -591,14 +595,17 @@ class HipOps:
             return self._linear_rows(x, gated, y, M, 2 * m.inter, K, 1)
         return self.swiglu(self.linear(x, m))
 
-    def swiglu(self, gu: torch.Tensor) -> torch.Tensor:
+    def swiglu(self, gu: torch.Tensor, limit: float = 0.0, slope: float = 1.0) -> torch.Tensor:
+        """From gate and up sums side by side [rows, 2 n] to the hidden units [rows, n]: silu(g) * u, or with a
+        positive ``limit`` the limited form g' * sigmoid(slope * g') * (u' + 1), g' = min(g, limit), u' = clamp(u,
+        -limit, limit)."""
         rows, two = gu.shape
         if two % 2:
             raise KernelError("swiglu input must hold gate and up side by side")
         self._want(gu, "swiglu input")
         out = torch.empty((rows, two // 2), dtype=gu.dtype, device=self.device)
         self._call(self.lib.tli_swiglu, gu.data_ptr(), out.data_ptr(), rows, two // 2,
-                   _dtype_code(gu.dtype), self._stream())
+                   _dtype_code(gu.dtype), float(limit), float(slope), self._stream())
         return out
 
     def qkv_to_cache(self, qkv, step, cache, heads, kv_heads, head_dim, q_norm, k_norm, rotary, queries=True):
@@ -1227,11 +1234,12 @@ class HipOps:
                    self.ROUTER_GROUP_SCORES.index(group_score), 1 if normalize else 0, _ptr(correction), self._stream())
         return ids, weights, gate
 
-    def apply_experts(self, x, ids, weights, w_gate_up, w_down, packed, shared, shared_gate):
+    def apply_experts(self, x, ids, weights, w_gate_up, w_down, packed, shared, shared_gate, limit=0.0, slope=1.0):
         """sum_j weights[t, j] * expert ids[t, j] (x[t])  (+ shared_gate[t] * shared[t], or + shared[t] without a
         gate);  ``w_gate_up`` [E, 2 ff, n] (an expert's gate rows, then its up rows), ``w_down`` [E, n, ff]; with
         ``packed`` (what ``pack_experts`` gave) the row-major matrices may be None.  An id from E on is an expert
-        that hands its input on: its term is weights[t, j] * x[t]."""
+        that hands its input on: its term is weights[t, j] * x[t].  ``limit`` > 0: the experts' hidden units are the
+        limited form (see ``swiglu``) instead of silu(gate) * up."""
         T, n = x.shape
         top = ids.shape[1]
         self._want(x, "expert input")
@@ -1268,7 +1276,7 @@ class HipOps:
                            pos.data_ptr(), tile_expert.data_ptr(), num_tiles.data_ptr(), hid.data_ptr(), part.data_ptr(),
                            None if shared is None else shared[t0:t1].data_ptr(),
                            None if (shared is None or shared_gate is None) else shared_gate[t0:t1].data_ptr(),
-                           out[t0:t1].data_ptr(), t1 - t0, top, E, n, ff, RT, self._stream())
+                           out[t0:t1].data_ptr(), t1 - t0, top, E, n, ff, RT, float(limit), float(slope), self._stream())
             return out
         if w_gate_up is None or w_down is None:
             raise KernelError("the experts' row-major matrices were not kept and the tiled ones do not apply here")
@@ -1283,7 +1291,8 @@ class HipOps:
                        w_gate_up.data_ptr(), w_down.data_ptr(), hid[t0 * top:].data_ptr(),
                        None if shared is None else shared[t0:t1].data_ptr(),
                        None if (shared is None or shared_gate is None) else shared_gate[t0:t1].data_ptr(),
-                       out[t0:t1].data_ptr(), t1 - t0, top, n, ff, E, _dtype_code(x.dtype), self._stream())
+                       out[t0:t1].data_ptr(), t1 - t0, top, n, ff, E, _dtype_code(x.dtype), float(limit), float(slope),
+                       self._stream())
         return out
 
     # ---- blocks that norm what a sublayer gives ------------------------------------------------------------
@@ -1326,11 +1335,13 @@ class HipOps:
             raise KernelError("a block table is narrower than its sequence needs")
 
     def sized_attention(self, q, step, g, kc, vc, heads, kv_heads, maps, key_dim, value_dim, scale, window, keep_first,
-                        out_dtype):
+                        out_dtype, sinks=None):
         """Attention of ``q`` [T, heads * maps, key_dim] over the key cache ``kc`` [pages, kv_heads * maps, page, key_dim]
         and the value cache ``vc`` [pages, kv_heads, value_dim, page] (None: a key's first value_dim elements are its
         values); map m of head h reads key head (h // (heads / kv_heads)) * maps + m.  A row at p sees t <= p with
-        p - t < window or t < keep_first (window None: all).  Returns [T, heads * maps, value_dim] of ``out_dtype``."""
+        p - t < window or t < keep_first (window None: all).  ``sinks`` (float32 [heads * maps]): the softmax's
+        denominator of (head, map) also holds exp(sink), a logit with no key and no value.  Returns [T, heads * maps,
+        value_dim] of ``out_dtype``."""
         T = step.num_rows
         self.check_sized_attention(heads, kv_heads, key_dim, value_dim)
         self._want(q, "queries", None, (T, heads * maps, key_dim))
@@ -1341,6 +1352,8 @@ class HipOps:
         elif value_dim > key_dim:
             raise KernelError("values that are the start of their keys cannot be longer than the keys")
         self._check_tables(g, step)
+        if sinks is not None:
+            self._want(sinks, "sinks", torch.float32, (heads * maps,))
         if out_dtype not in (q.dtype, torch.float32):
             raise KernelError(f"attention over {q.dtype} gives {q.dtype} or float32, not {out_dtype}")
         out = torch.empty((T, heads * maps, value_dim), dtype=out_dtype, device=self.device)
@@ -1354,12 +1367,12 @@ class HipOps:
             self._call(self.lib.tli_attention_sized_mfma_bf16, q.data_ptr(), out.data_ptr(), kc.data_ptr(), _ptr(vc),
                        step.row_start.data_ptr(), step.seq_start.data_ptr(), step.num_seqs, tiles, g.tables.data_ptr(),
                        g.table_width, g.page_size, pages, heads, kv_heads, maps, key_dim, value_dim, float(scale),
-                       int(window or 0), keep, grouped, 1 if out_dtype == torch.float32 else 0, self._stream())
+                       int(window or 0), keep, grouped, 1 if out_dtype == torch.float32 else 0, _ptr(sinks), self._stream())
             return out
         self._call(self.lib.tli_attention_sized_plain, q.data_ptr(), out.data_ptr(), kc.data_ptr(), _ptr(vc),
                    step.positions.data_ptr(), step.seq_of_row.data_ptr(), g.tables.data_ptr(), g.table_width, g.page_size,
                    pages, T, heads, kv_heads, maps, key_dim, value_dim, float(scale), int(window or 0),
-                   keep, _dtype_code(q.dtype), 1 if out_dtype == torch.float32 else 0,
+                   keep, _dtype_code(q.dtype), 1 if out_dtype == torch.float32 else 0, _ptr(sinks),
                    self._stream())
         return out
 
@@ -1420,13 +1433,13 @@ class HipOps:
         return out
 
     def latent_attention(self, proj, step, cache, heads, dim, rot, rank, vdim, norm_weight, norm_eps, rotary, scale,
-                         w_qk, w_v):
+                         w_qk, w_v, sinks=None):
         """Attention whose keys and values are made from one latent vector a position, from the raw projections
         ``proj`` [T, q (heads * (dim + rot)) | latent (rank) | key part (rot)] to the heads' outputs [T, heads * vdim].
         The cache (record "latent" [page, rank + rot]) keeps the normed latent vector and the turned key part; a
         head's score is q_plain . (W_uk c) + q_turned . k_turned, computed as (W_uk^T q_plain) . c with ``w_qk``
         [heads, rank, dim] = W_uk^T a head, so that all heads read the one cached vector; the weighted sum of the
-        latent vectors then goes through ``w_v`` [heads, vdim, rank] = W_uv a head."""
+        latent vectors then goes through ``w_v`` [heads, vdim, rank] = W_uv a head.  ``sinks``: as in ``sized_attention``."""
         T = step.num_rows
         width = heads * (dim + rot) + rank + rot
         self._want(proj, "projections", None, (T, width))
@@ -1450,8 +1463,93 @@ class HipOps:
         self._want(w_v, "matrices out of the latent space", proj.dtype, (heads, vdim, rank))
         self.head_products(proj, dim + rot, w_qk, out=q.view(T, heads * key), out_stride=key)
         o = self.sized_attention(q, step, g, kc.view(pages, 1, g.page_size, key), None, heads, 1, 1, key, rank, scale,
-                                 None, 0, proj.dtype)
+                                 None, 0, proj.dtype, sinks=sinks)
         return self.head_products(o.view(T, heads * rank), rank, w_v)
+
+    # ---- attention with biases and a sink whose values may be its keys ------------------------------------
+    def sink_attention(self, proj, step, cache, heads, kv_heads, head_dim, bias, rotary, scale, sinks, window,
+                       values_are_keys):
+        """From the raw projections ``proj`` [T, q (heads * head_dim) | k (kv_heads * head_dim) (| v likewise, unless
+        ``values_are_keys``)] to the heads' outputs [T, heads * head_dim]: ``bias`` (float32 over the projections' row,
+        or None) is added, q and k are turned (``rotary``: cos, sin, turned elements; pairs (i, i + n/2)), the turned
+        keys and the values (the keys before they are turned, or their own projection) go into the cache (records
+        "k" [kv_heads, page, head_dim] and "v" [kv_heads, head_dim, page]), attention with ``sinks`` (float32 [heads]
+        or None) over the cache."""
+        T = step.num_rows
+        width = (heads + (1 if values_are_keys else 2) * kv_heads) * head_dim
+        self._want(proj, "projections", None, (T, width))
+        if bias is not None:
+            self._want(bias, "projections' bias", torch.float32, (width,))
+        if cache is None or not cache.writes:
+            raise KernelError("this attention writes its keys and values into a cache layer of its own")
+        kc, vc, g = cache.record("k"), cache.record("v"), cache.group
+        self._check_cache(kc, vc, g, kv_heads, head_dim, proj.dtype, step)
+        cos = sin = None
+        rd = npos = 0
+        if rotary is not None:
+            cos, sin, rd = self._rotary(rotary, step)
+            npos = cos.shape[0]
+        q = torch.empty((T, heads, head_dim), dtype=proj.dtype, device=self.device)
+        self._call(self.lib.tli_keyed_prepare, proj.data_ptr(), width, _ptr(bias), q.data_ptr(), kc.data_ptr(), vc.data_ptr(),
+                   step.positions.data_ptr(), step.seq_of_row.data_ptr(), g.tables.data_ptr(), g.table_width, g.page_size,
+                   kc.shape[0], T, heads, kv_heads, head_dim, -1 if values_are_keys else (heads + kv_heads) * head_dim,
+                   _ptr(cos), _ptr(sin), rd, npos, _dtype_code(proj.dtype), self._stream())
+        o = self.sized_attention(q, step, g, kc, vc, heads, kv_heads, 1, head_dim, head_dim, scale, window, 0, proj.dtype,
+                                 sinks=sinks)
+        return o.view(T, heads * head_dim)
+
+    def add_bias(self, y, bias):
+        """y [T, n] += bias (float32 [n]), in place; ``y`` may be an unfinished product."""
+        y = self.resolve(y)
+        T, n = y.shape
+        self._want(y, "rows")
+        self._want(bias, "bias", torch.float32, (n,))
+        self._call(self.lib.tli_add_bias, y.data_ptr(), bias.data_ptr(), T, n, _dtype_code(y.dtype), self._stream())
+        return y
+
+    # ---- lightning attention -----------------------------------------------------------------------------
+    def check_lightning_sizes(self, heads: int, dk: int, dv: int) -> None:
+        if heads <= 0 or not 1 <= dk <= 256 or dv < 1:
+            raise KernelError(f"lightning attention with {heads} heads of keys of {dk} (1 to 256) and values of {dv} is not supported")
+
+    def lightning_state_shape(self, heads: int, dk: int, dv: int):
+        """The shape of one request's recurrent state (float32): a head's matrix is kept transposed, so that the
+        elements of a column, which one DPP row of lanes holds, lie together."""
+        return (heads, dv, dk)
+
+    def lightning_attention(self, proj, decay, state, step, heads, dk, dv):
+        """From the raw projections ``proj`` [T, >= q (H dk) | k (H dk) | v (H dv)] to the heads' outputs of the
+        recurrence S <- decay_h S + silu(k) silu(v)^T, o = S^T silu(q), float32 [T, H dv].  ``decay``: float32 [H];
+        ``state``: float32 [slots, H, dv, dk], read (unless a sequence starts at position 0) and replaced."""
+        T = step.num_rows
+        self.check_lightning_sizes(heads, dk, dv)
+        need = 2 * heads * dk + heads * dv
+        if proj.dim() != 2 or proj.shape[0] != T or proj.shape[1] < need:
+            raise KernelError(f"the projections have shape {tuple(proj.shape)}, expected [{T}, >= {need}]")
+        self._want(proj, "projections")
+        self._want(decay, "decays", torch.float32, (heads,))
+        self._want(state, "recurrent state", torch.float32, (state.shape[0], heads, dv, dk))
+        if max(step.h_slots, default=0) >= state.shape[0]:
+            raise KernelError("a sequence's slot lies outside the state")
+        out = torch.empty((T, heads * dv), dtype=torch.float32, device=self.device)
+        self._call(self.lib.tli_lightning_recurrence, proj.data_ptr(), proj.shape[1], decay.data_ptr(), state.data_ptr(),
+                   out.data_ptr(), step.row_start.data_ptr(), step.seq_start.data_ptr(), step.slots.data_ptr(),
+                   step.num_seqs, heads, dk, dv, _dtype_code(proj.dtype), self._stream())
+        return out
+
+    def lightning_norm(self, o, proj, gate_at, weight, eps, out_dtype):
+        """y = o / sqrt(mean(o^2) + eps) * weight * sigmoid(gate) over a whole row; ``o`` float32 [T, n], the gate's
+        logits are columns ``gate_at`` .. ``gate_at + n`` of ``proj``."""
+        T, n = o.shape
+        self._want(o, "heads' outputs", torch.float32)
+        self._want(proj, "projections", out_dtype)
+        if proj.shape[0] != T or proj.shape[1] < gate_at + n:
+            raise KernelError("the gate lies outside the projections")
+        self._want(weight, "norm weight", torch.float32, (n,))
+        out = torch.empty((T, n), dtype=out_dtype, device=self.device)
+        self._call(self.lib.tli_lightning_norm, o.data_ptr(), proj.data_ptr() + gate_at * proj.element_size(), proj.shape[1],
+                   weight.data_ptr(), out.data_ptr(), T, n, float(eps), _dtype_code(out_dtype), self._stream())
+        return out
 
     def sample(self, logits: torch.Tensor, temperatures: Optional[torch.Tensor] = None,
                seeds: Optional[torch.Tensor] = None, top_p: Optional[torch.Tensor] = None) -> torch.Tensor:

@@ -3,3 +3,4 @@ from . import qwen3  # noqa: F401
 from . import sinepel  # noqa: F401
 from . import kapanex  # noqa: F401
 from . import gimipel  # noqa: F401
+from . import defosun  # noqa: F401

@@ -1,4 +1,4 @@
-from . import attention, block, conv_attention, delta, differential, latent, postnorm, embedding, hyper, mlp, moe, norm, parallel, rope  # noqa: F401  (registers the parts)
+from . import attention, block, conv_attention, delta, differential, latent, lightning, postnorm, sink_attention, embedding, hyper, mlp, moe, norm, parallel, rope  # noqa: F401  (registers the parts)
 from .base import (Block, BuildEnv, FeedForward, GroupView, LayerCache, Mixer, Norm, Part,
                    PositionEncoding, RotaryTables, StepView, build_part, register_part)
 

@@ -12,6 +12,9 @@ beside an optional shared one that every row uses.
         names no gate for the shared expert)
     expert(h) = W_down (silu(W_gate h) * (W_up h));  the last I (``identity``) router outputs stand for
         experts without matrices whose output is h itself
+    ``activation`` "limited": an expert's hidden units are g * sigmoid(slope * g) * (u + 1) with
+        g = min(W_gate h, limit), u = clamp(W_up h, -limit, limit)  (``limit``, ``gate_slope``; the shared
+        expert with ``shared_limit``)
 
 The router's product gives float32 (the row of the shared expert's gate rides along as one more
 row of that matrix); scores, choice and weights are float32.  A row's chosen experts are added
@@ -25,7 +28,7 @@ import torch
 
 from ..weights.loader import TensorDecl
 from .base import BuildEnv, FeedForward, StepView, register_part
-from .linear import GatedMatrix, as_matrix
+from .linear import GatedMatrix, as_matrix, fuse_rows
 
 
 class RoutedExperts(FeedForward):
@@ -51,6 +54,14 @@ class RoutedExperts(FeedForward):
         if self.experts < 1 or self.outputs % self.groups or not 1 <= self.keep <= self.groups \
                 or not 1 <= self.top <= self.keep * (self.outputs // self.groups):
             raise ValueError(f"{self.outputs} router outputs in {self.groups} groups, {self.keep} kept, cannot give {self.top}")
+        self.activation = str(p.get("activation", "silu"))
+        if self.activation not in ("silu", "limited"):
+            raise ValueError(f"activation '{self.activation}' is not known; known: silu, limited")
+        self.limit = float(p.get("limit", 0.0)) if self.activation == "limited" else 0.0
+        self.shared_limit = float(p.get("shared_limit", self.limit)) if self.activation == "limited" else 0.0
+        self.slope = float(p.get("gate_slope", 1.0))
+        if self.activation == "limited" and (self.limit <= 0.0 or self.shared_limit <= 0.0):
+            raise ValueError("the limited activation needs a positive limit")
         self.correction_name = spec.names.get("correction")
         self.shared_gated = "shared_scale" in spec.names
 
@@ -97,7 +108,10 @@ class RoutedExperts(FeedForward):
             self.w_gate_up = self.w_down = None
         self.shared_gate_up = self.shared_down = None
         if self.shared_inter is not None:
-            self.shared_gate_up = GatedMatrix(weights[n["shared_gate"]], weights[n["shared_up"]], env)
+            if self.activation == "silu":
+                self.shared_gate_up = GatedMatrix(weights[n["shared_gate"]], weights[n["shared_up"]], env)
+            else:       # (the products' own epilogue is silu(gate) * up: gate and up rows stacked, the activation in a pass of its own)
+                self.shared_gate_up = fuse_rows([weights[n["shared_gate"]], weights[n["shared_up"]]], env)
             self.shared_down = as_matrix(weights[n["shared_down"]], env)
 
     def workspace_elems(self, rows: int) -> int:
@@ -113,8 +127,13 @@ class RoutedExperts(FeedForward):
                                                       self.has_gate, transposed, **how)
         shared = None
         if self.shared_inter is not None:
-            shared = ops.linear(ops.linear_swiglu(x, self.shared_gate_up), self.shared_down)
-        return ops.apply_experts(x, ids, weights, self.w_gate_up, self.w_down, self.packed, shared, shared_gate)
+            if self.activation == "silu":
+                hidden = ops.linear_swiglu(x, self.shared_gate_up)
+            else:
+                hidden = ops.swiglu(ops.linear(x, self.shared_gate_up), limit=self.shared_limit, slope=self.slope)
+            shared = ops.linear(hidden, self.shared_down)
+        how = {} if self.activation == "silu" else {"limit": self.limit, "slope": self.slope}
+        return ops.apply_experts(x, ids, weights, self.w_gate_up, self.w_down, self.packed, shared, shared_gate, **how)
 
 
 register_part("ffn", "routed_experts", RoutedExperts)

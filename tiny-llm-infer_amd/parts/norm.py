@@ -1,6 +1,8 @@
 """RMSNorm: y_j = w_j * x_j / sqrt(mean(x^2) + eps), all in float32
 (kernels/src/rmsnorm_kernel_cpu.cpp:27-43).  The weight is a plain multiplier; a
-norm whose spec names no weight has none (all ones).
+norm whose spec names no weight has none (all ones).  ``weight_offset`` c: the checkpoint stores
+the multiplier less c (a weight kept around zero is ``weight_offset`` 1), added in float32 when
+the weight is loaded.
 The residual stream is float32; the norm adds what the previous part owes the
 residual before it normalises, so the residual sum is never rounded.
 
@@ -26,10 +28,12 @@ class RMSNorm(Norm):
         self.size = int(spec.params["size"])
         self.eps = float(spec.params["eps"])
         self.weight_name = spec.names.get("weight")             # None: a norm without weights
+        self.offset = float(spec.params.get("weight_offset", 0.0))
         self.weight: Optional[torch.Tensor] = None
 
     def tensors(self) -> List[TensorDecl]:
-        return [TensorDecl(self.weight_name, (self.size,), "ones_normal")] if self.weight_name is not None else []
+        init = "ones_normal" if self.offset == 0.0 else f"normal({1.0 - self.offset},0.02)"
+        return [TensorDecl(self.weight_name, (self.size,), init)] if self.weight_name is not None else []
 
     def load(self, weights: Dict[str, torch.Tensor], env: BuildEnv) -> None:
         super().load(weights, env)
@@ -38,6 +42,8 @@ class RMSNorm(Norm):
             self.weight = torch.ones(self.size, dtype=torch.float32, device=env.device)
         else:
             self.weight = weights[self.weight_name].to(torch.float32).contiguous()
+            if self.offset != 0.0:
+                self.weight = (self.weight + self.offset).contiguous()
 
     def as_rms(self):
         return self.weight, self.eps

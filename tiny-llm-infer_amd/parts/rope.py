@@ -7,6 +7,9 @@ exponent -2.0f*i/d in float32; angle = float32(position) * f_i in float32
 (kernels/src/rope_kernel_cpu.cpp:156-179).  ``rotary_dim`` = d may be smaller
 than the head size; the rest of the head is left as it is.  The table holds
 sin and cos of the float32 angle, evaluated in float64 and rounded once.
+
+"rope_interleaved" is the same table for an encoding whose pair i is the neighbours
+(2i, 2i + 1); the mixer that applies it is told so by ``RotaryTables.pairing``.
 """
 from __future__ import annotations
 
@@ -52,4 +55,10 @@ class NeoxRope(PositionEncoding):
         return RotaryTables(self.cos, self.sin, self.rotary_dim, "half")
 
 
+class InterleavedRope(NeoxRope):
+    def rotary(self) -> RotaryTables:
+        return RotaryTables(self.cos, self.sin, self.rotary_dim, "interleaved")
+
+
 register_part("position", "rope_neox", NeoxRope)
+register_part("position", "rope_interleaved", InterleavedRope)
