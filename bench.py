@@ -66,14 +66,14 @@ DESIGN_SIZES = {
 
 
 def compare_designs(args):
-    """Prefill and decode of the Sinepel design (or, with --design-names, of others: Kapanex, Gimipel) beside the Qwen3
+    """Prefill and decode of the Sinepel design (or, with --design-names, of others: Kapanex, Gimipel, Defosun) beside the Qwen3
     dense decoder at equal layer sizes
     (random bfloat16 weights, 4 layers unless --layers says otherwise), through the step function:
     one prompt of --prefill-tokens in one step, and decode steps of --batch and 64 requests at
     --prompt-len tokens of context.  One JSON line."""
     import torch
 
-    from tiny_llm_infer_amd.config import GimipelConfig, KapanexConfig, Qwen3Config, SinepelConfig
+    from tiny_llm_infer_amd.config import DefosunConfig, GimipelConfig, KapanexConfig, Qwen3Config, SinepelConfig
     from tiny_llm_infer_amd.engine.loading import random_model
     from tiny_llm_infer_amd.engine.runner import ModelRunner, StepEntry
     import random
@@ -129,8 +129,23 @@ def compare_designs(args):
                         "mixer": {"heads": heads, "dim": dim, "rot_dim": dim // 2, "vdim": dim, "kv_rank": 4 * dim,
                                   "scale": (dim + dim // 2) ** -0.5, "rot": {"dims": dim // 2, "base": 1e6}}}
                        for i in range(layers)]})
+        # Defosun: four streams; attention whose values are its keys (heads as Qwen3's, half of every head turned, a sink)
+        # with the dense feed-forward, latent attention (as Gimipel's, with a sink) and lightning attention (heads as
+        # Qwen3's, a state of dim x dim a head) in turn, the latter two with 16 experts of a quarter of the feed-forward
+        # size of which 2 are chosen beside a shared expert of half of it (the limited activation)
+        dmoe = {"kind": "moe", "expert": {"ff": ff // 4, "limit": 7.0}, "shared": {"ff": ff // 2, "limit": 7.0},
+                "router": {"experts": 16, "top": 2}}
+        dmixers = [("attention", {"heads": heads, "kv_heads": kv_heads, "dim": dim, "vdim": dim, "scale": dim ** -0.5,
+                                  "rot": {"dims": dim // 2, "base": 1e6}}, {"kind": "dense", "ff": ff}),
+                   ("latent_attention", {"heads": heads, "dim": dim, "rot_dim": dim // 2, "vdim": dim, "kv_rank": 4 * dim,
+                                         "scale": (dim + dim // 2) ** -0.5, "rot": {"dims": dim // 2, "base": 1e6}}, dmoe),
+                   ("lightning", {"heads": heads, "dim": dim, "vdim": dim,
+                                  "decay": [1.0 - 2.0 ** (-1 - 8 * h / heads) for h in range(heads)]}, dmoe)]
+        defosun = DefosunConfig.from_dict({
+            "architecture": "Defosun", "vocab": vocab, "width": width, "norm": {"eps": 1e-5}, "streams": 4, "max_positions": context,
+            "layers": [{"type": dmixers[i % 3][0], "mixer": dmixers[i % 3][1], "mlp": dmixers[i % 3][2]} for i in range(layers)]})
         known = {"sinepel": ("Sinepel", sinepel), "kapanex": ("Kapanex", kapanex), "gimipel": ("Gimipel", gimipel),
-                 "qwen3": ("Qwen3ForCausalLM", qwen)}
+                 "defosun": ("Defosun", defosun), "qwen3": ("Qwen3ForCausalLM", qwen)}
         names = [n for n in args.design_names.split(",") if n]
         if any(n not in known for n in names):
             print(f"--design-names: known designs are {', '.join(known)}")
@@ -211,7 +226,7 @@ def main():
                     help="instead of the default workload: the Sinepel design beside the Qwen3 dense decoder at equal layer "
                          f"sizes, prefill and decode; a list of {','.join(DESIGN_SIZES)} or 'all'")
     ap.add_argument("--design-names", default="sinepel,qwen3",
-                    help="with --designs: which designs are run at every size (sinepel, kapanex, gimipel, qwen3)")
+                    help="with --designs: which designs are run at every size (sinepel, kapanex, gimipel, defosun, qwen3)")
     args = ap.parse_args()
     if args.gpus != 1:
         print(f"bench.py runs on one GPU only; --gpus {args.gpus} is not supported (single-GPU engine)")

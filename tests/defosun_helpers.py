@@ -78,7 +78,7 @@ SMALL = {
 
 
 def make_weights(cfg: dict, seed: int, clear_routing: bool = False, mild: bool = False) -> Dict[str, torch.Tensor]:
-    """bfloat16 weights of a size that makes every mechanism show in the logits.  ``mild``: queries half as large,
+    """bfloat16 weights of a size that makes every mechanism show in the logits.  ``mild``: queries and keys half as large,
     so that a softmax does not multiply the rounding of bfloat16 queries and keys.  ``clear_routing``: no router's
     choice depends on anything that rounding touches, so that a run in bfloat16 chooses as the plain
     implementation does (a row that goes to another expert is another computation).  The last n elements of the
@@ -101,7 +101,7 @@ def make_weights(cfg: dict, seed: int, clear_routing: bool = False, mild: bool =
             H, G, d = m["heads"], m["kv_heads"], m["dim"]
             w[p + "mix.q"] = normal(H * d, D, std=D ** -0.5 * 3 * sharp)
             w[p + "mix.q.b"] = normal(H * d, std=0.3)
-            w[p + "mix.k"] = normal(G * d, D, std=D ** -0.5 * 2)
+            w[p + "mix.k"] = normal(G * d, D, std=D ** -0.5 * 2 * sharp)
             w[p + "mix.k.b"] = normal(G * d, std=0.3)
             w[p + "mix.sink"] = normal(H, std=1.0, mean=1.0)
             w[p + "mix.o"] = normal(D, H * d, std=(H * d) ** -0.5 * 1.5)
@@ -111,7 +111,7 @@ def make_weights(cfg: dict, seed: int, clear_routing: bool = False, mild: bool =
             w[p + "mix.q"] = normal(H * (d + r), D, std=D ** -0.5 * 3 * sharp)
             w[p + "mix.dkv"] = normal(n + r, D, std=D ** -0.5 * 2)
             w[p + "mix.dkv.norm"] = normal(n, std=0.1, mean=1.0)
-            w[p + "mix.uk"] = normal(H * d, n, std=n ** -0.5 * 2)
+            w[p + "mix.uk"] = normal(H * d, n, std=n ** -0.5 * 2 * sharp)
             w[p + "mix.uv"] = normal(H * e, n, std=n ** -0.5 * 1.5)
             w[p + "mix.sink"] = normal(H, std=1.0, mean=1.0)
             w[p + "mix.o"] = normal(D, H * e, std=(H * e) ** -0.5 * 1.5)

@@ -229,7 +229,7 @@ def test_streams_around_a_dense_feed_forward(tmp_path, dtype, streams):
     cfg = _config(90, 48, [_layer("attention", _attention(2, 1, 16, 16), _dense(72))] * 2, streams=streams)
     folder = write_folder(str(tmp_path / "streams"), cfg, make_weights(cfg, 10 + streams, mild=True))
     reqs = _requests(90, [50, 3, 77], seed=8)
-    _all_cuts(folder, dtype, reqs, plain_logits(folder, reqs), 8, 192, TOL[dtype], f"{streams} streams")
+    _all_cuts(folder, dtype, reqs, plain_logits(folder, reqs), 8, 128, TOL[dtype], f"{streams} streams")
 
 
 # ---------------------------------------------- a key far back, at the borders of pages; the sink ---
