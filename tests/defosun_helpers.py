@@ -146,7 +146,7 @@ def make_weights(cfg: dict, seed: int, clear_routing: bool = False, mild: bool =
             for q in (1, 2) if f is not None else (1,):
                 w[f"{p}hc{q}.in"] = normal(S, std=0.1, mean=1.0 / S)
                 w[f"{p}hc{q}.out"] = normal(S, std=0.15, mean=0.6)
-                w[f"{p}hc{q}.mix"] = torch.eye(S) * 0.8 + normal(S, S, std=0.1).abs()
+                w[f"{p}hc{q}.mix"] = torch.eye(S) * (1.0 if S == 1 else 0.8) + normal(S, S, std=0.1).abs()      # (one stream: nothing else keeps the embedding)
     if clear_routing:
         n = max([layer["mlp"]["router"]["experts"] for layer in cfg["layers"]
                  if layer["mlp"] is not None and layer["mlp"]["kind"] == "moe"], default=0)
