@@ -145,10 +145,13 @@ def test_experts_with_the_limited_activation(ops, dtype, T, E, top, n, ff, limit
 
 
 @pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
-@pytest.mark.parametrize("heads, dk, dv", [(2, 16, 24), (3, 20, 12), (1, 40, 20), (4, 64, 32), (2, 128, 128), (1, 200, 50), (5, 8, 7)])
-def test_lightning_recurrence_in_portions_and_slots_that_are_used_again(ops, dtype, heads, dk, dv):
+@pytest.mark.parametrize("lanes", [16, 64])
+@pytest.mark.parametrize("heads, dk, dv", [(2, 16, 24), (3, 20, 12), (1, 40, 20), (4, 64, 32), (2, 128, 128), (1, 200, 50), (5, 8, 7),
+                                           (1, 256, 16)])
+def test_lightning_recurrence_in_portions_and_slots_that_are_used_again(ops, dtype, heads, dk, dv, lanes, monkeypatch):
     """Three sequences cut into portions of 1 to 43 rows side by side, in slots that are never cleared and are
-    used again by the next sequences; decays from 0.5 to 1."""
+    used again by the next sequences; decays from 0.5 to 1; a column of the state in 16 lanes and in 64."""
+    monkeypatch.setattr(ops, "lightning_lanes", lanes)
     g = torch.Generator().manual_seed(dk * dv)
     dt = DTYPES[dtype]
     decay = torch.linspace(0.5, 1.0, heads)

@@ -8,17 +8,17 @@
 // lie together), so that a wave reads and writes it in runs.  A sequence that starts at position 0 does not read its
 // slot: slots are never cleared when they change hands.
 //
-// Columns of S are independent.  A workgroup takes LT_COLS columns of one head of one sequence and walks the
-// sequence's rows in order; a column belongs to the 16 lanes of a DPP row, lane s holding elements s R .. s R + R - 1
-// of it in registers (R = dk / 16 rounded up to a power of two; elements from dk on stay zero).  A row costs R
-// multiply-adds for the state, R for the output and four DPP moves.  The rows come through LDS in chunks that the
-// whole workgroup fetches (with the silu) into registers while the chunk before is walked.
+// Columns of S are independent.  A workgroup takes a few columns of one head of one sequence and walks the
+// sequence's rows in order; a column belongs to the 16 lanes of a DPP row (a workgroup then has 16 columns), or to
+// the 64 lanes of a wave (4 columns), lane s holding elements s R .. s R + R - 1 of it in registers (R = dk / lanes
+// rounded up to a power of two; elements from dk on stay zero).  A row costs R multiply-adds for the state, R for
+// the output and four DPP moves (and two exchanges of rows of lanes, with 64 lanes a column).  The rows come through LDS in chunks that the
+// whole workgroup fetches into registers while the chunk before is walked (the silu is taken on their way into LDS).
 //
 // lightning_norm: y = o / sqrt(mean(o^2) + eps) * w * sigmoid(gate) over all heads of a row together.
 #include "common.h"
 
 #define LT_THREADS 256
-#define LT_COLS 16
 #define LT_MAX_DK 256
 
 __device__ __forceinline__ float lt_silu(float z) { return z / (1.0f + expf(-z)); }
@@ -32,34 +32,44 @@ __device__ __forceinline__ float lt_sum16(float v) {
     return v;
 }
 
-template <typename T, int R, int CH>
+// L lanes a column (16 or 64), R elements of it a lane, CH rows a chunk
+template <typename T, int L, int R, int CH>
 __global__ __launch_bounds__(LT_THREADS) void lightning_recurrence_kernel(
     const T* __restrict__ proj, int ld, const float* __restrict__ decay, float* __restrict__ state,
     float* __restrict__ out, const int* __restrict__ row_start, const int* __restrict__ seq_start,
     const int* __restrict__ slots, int H, int dk, int dv) {
-    constexpr int DKP = 16 * R;
-    constexpr int W = 2 * DKP + LT_COLS;                 // floats of a staged row: q, k, the workgroup's values
+    constexpr int DKP = L * R;
+    constexpr int NC = LT_THREADS / L;                   // columns a workgroup
+    constexpr int W = 2 * DKP + 16;                      // floats of a staged row: q, k, the workgroup's values (up to 16)
     constexpr int PF = CH * W / LT_THREADS;
-    static_assert(PF * LT_THREADS == CH * W, "a chunk is shared out evenly");
+    constexpr int VW = R % 4 == 0 ? 4 : R % 2 == 0 ? 2 : 1;   // floats a piece of the state that a lane moves at once
+    static_assert(PF * LT_THREADS == CH * W && PF <= 64 && NC <= 16, "a chunk is shared out evenly");
     __shared__ __align__(16) float rows_s[CH * W];
-    const int seq = blockIdx.z, h = blockIdx.y, j0 = blockIdx.x * LT_COLS;
-    const int tid = threadIdx.x, lane = tid % TLI_WAVE, wave = tid / TLI_WAVE;
-    const int sub = lane % 16, jl = wave * 4 + lane / 16;
+    const int seq = blockIdx.z, h = blockIdx.y, j0 = blockIdx.x * NC;
+    const int tid = threadIdx.x;
+    const int sub = tid % L, jl = tid / L;
     const int j = j0 + jl;
     const int r0 = row_start[seq], n = row_start[seq + 1] - r0;
     if (n <= 0) return;
     const float lam = decay[h];
     float* col = state + (((size_t)slots[seq] * H + h) * dv + (j < dv ? j : 0)) * dk;
-    const bool whole = dk == DKP && R % 4 == 0;          // the lane's elements as 16-byte pieces
+    const bool whole = dk == DKP && dk % 4 == 0;         // every lane's elements exist, and its pieces are aligned
     float S[R];
 #pragma unroll
     for (int r = 0; r < R; ++r) S[r] = 0.f;
     if (seq_start[seq] != 0 && j < dv) {
         if (whole) {
 #pragma unroll
-            for (int r = 0; r < R / 4 * 4; r += 4) {
-                const float4 v = *reinterpret_cast<const float4*>(col + sub * R + r);
-                S[r] = v.x, S[r + 1] = v.y, S[r + 2] = v.z, S[r + 3] = v.w;
+            for (int r = 0; r < R; r += VW) {
+                if constexpr (VW == 4) {
+                    const float4 v = *reinterpret_cast<const float4*>(col + sub * R + r);
+                    S[r] = v.x, S[r + 1] = v.y, S[r + 2] = v.z, S[r + 3] = v.w;
+                } else if constexpr (VW == 2) {
+                    const float2 v = *reinterpret_cast<const float2*>(col + sub * R + r);
+                    S[r] = v.x, S[r + 1] = v.y;
+                } else {
+                    S[r] = col[sub * R + r];
+                }
             }
         } else {
 #pragma unroll
@@ -68,24 +78,24 @@ __global__ __launch_bounds__(LT_THREADS) void lightning_recurrence_kernel(
         }
     }
     const size_t q_at = (size_t)h * dk, k_at = (size_t)H * dk + (size_t)h * dk, v_at = (size_t)2 * H * dk + (size_t)h * dv;
-    float pf[PF];
+    // A chunk's elements are fetched as they lie in memory, every load issued before any is used: which element a
+    // thread takes (its row of the chunk, its column of q, k or v) is arithmetic on constants; an element that does
+    // not exist (past the sequence's end, past dk or dv) is not loaded (where none of a wave's exist, the wave leaves
+    // the load out) or dropped when the chunk is written into LDS, where the silu is taken too.
+    T raw[PF];
+    unsigned long long live = 0;
     auto fetch = [&](int first) {
+        live = 0;
 #pragma unroll
         for (int u = 0; u < PF; ++u) {
             const int e = tid + u * LT_THREADS;
-            const int t = first + e / W, cc = e % W;
-            float val = 0.f;
-            if (t < n) {
-                const T* src = proj + (size_t)(r0 + t) * ld;
-                if (cc < DKP) {
-                    if (cc < dk) val = lt_silu(to_f32(src[q_at + cc]));
-                } else if (cc < 2 * DKP) {
-                    if (cc - DKP < dk) val = lt_silu(to_f32(src[k_at + cc - DKP]));
-                } else if (j0 + cc - 2 * DKP < dv) {
-                    val = lt_silu(to_f32(src[v_at + j0 + cc - 2 * DKP]));
-                }
-            }
-            pf[u] = val;
+            const int rr = e / W, cc = e - rr * W;
+            const int i = cc < DKP ? cc : cc - DKP, jc = cc - 2 * DKP;
+            const size_t at = cc < DKP ? q_at + i : cc < 2 * DKP ? k_at + i : v_at + j0 + jc;
+            const bool ok = first + rr < n && (cc < 2 * DKP ? i < dk : (jc < NC && j0 + jc < dv));
+            raw[u] = 0;
+            if (__builtin_amdgcn_ballot_w64(ok)) raw[u] = proj[ok ? (size_t)(r0 + first + rr) * ld + at : (size_t)r0 * ld + q_at];
+            live |= (unsigned long long)ok << u;
         }
     };
     fetch(0);
@@ -93,10 +103,11 @@ __global__ __launch_bounds__(LT_THREADS) void lightning_recurrence_kernel(
     for (int t0 = 0; t0 < n; t0 += CH) {
         __syncthreads();                                 // the chunk before has been walked by every wave
 #pragma unroll
-        for (int u = 0; u < PF; ++u) rows_s[tid + u * LT_THREADS] = pf[u];
+        for (int u = 0; u < PF; ++u) rows_s[tid + u * LT_THREADS] = (live >> u & 1) ? lt_silu(to_f32(raw[u])) : 0.f;
         __syncthreads();
         if (t0 + CH < n) fetch(t0 + CH);
         const int cnt = min(CH, n - t0);
+#pragma unroll 4
         for (int t = 0; t < cnt; ++t) {
             const float* row = rows_s + t * W;
             const float v = row[2 * DKP + jl];
@@ -107,14 +118,18 @@ __global__ __launch_bounds__(LT_THREADS) void lightning_recurrence_kernel(
                 acc = fmaf(S[r], row[sub * R + r], acc);
             }
             acc = lt_sum16(acc);
+            if constexpr (L == 64) acc = quad_rows_sum(acc);
             if (sub == 0 && j < dv) o_col[(size_t)(t0 + t) * H * dv] = acc;
         }
     }
     if (j >= dv) return;
     if (whole) {
 #pragma unroll
-        for (int r = 0; r < R / 4 * 4; r += 4)
-            *reinterpret_cast<float4*>(col + sub * R + r) = make_float4(S[r], S[r + 1], S[r + 2], S[r + 3]);
+        for (int r = 0; r < R; r += VW) {
+            if constexpr (VW == 4) *reinterpret_cast<float4*>(col + sub * R + r) = make_float4(S[r], S[r + 1], S[r + 2], S[r + 3]);
+            else if constexpr (VW == 2) *reinterpret_cast<float2*>(col + sub * R + r) = make_float2(S[r], S[r + 1]);
+            else col[sub * R + r] = S[r];
+        }
     } else {
 #pragma unroll
         for (int r = 0; r < R; ++r)
@@ -123,27 +138,37 @@ __global__ __launch_bounds__(LT_THREADS) void lightning_recurrence_kernel(
 }
 
 // proj: [T, ld] raw projections, q (H dk), k (H dk), v (H dv) first; decay: float32 [H]; state: float32
-// [slots, H, dv, dk]; out: float32 [T, H dv]; row_start [seqs + 1], seq_start, slots [seqs]
+// [slots, H, dv, dk]; out: float32 [T, H dv]; row_start [seqs + 1], seq_start, slots [seqs].
+// lanes: 16 or 64 lanes a column, or 0: 64 where the sequences, heads and columns are too few to give every SIMD of
+// the chip two waves at 16 (one long prompt), else 16 (a wave then has four columns and a quarter of the additions
+// across lanes a column)
 extern "C" int tli_lightning_recurrence(const void* proj, int ld, const float* decay, float* state, float* out,
                                         const int* row_start, const int* seq_start, const int* slots, int seqs, int H,
-                                        int dk, int dv, int dtype, void* stream) {
+                                        int dk, int dv, int dtype, int lanes, void* stream) {
     if (seqs <= 0) return 0;
     if (H <= 0 || dk <= 0 || dv <= 0 || dk > LT_MAX_DK)
         return tli_fail("lightning: bad sizes (heads %d, keys of %d (at most %d), values of %d)", H, dk, LT_MAX_DK, dv);
     if (ld < 2 * H * dk + H * dv) return tli_fail("lightning: rows of %d hold fewer than q, k and v", ld);
     if (H > 65535 || seqs > 65535) return tli_fail("lightning: too many heads or sequences for one launch");
-    const dim3 grid((dv + LT_COLS - 1) / LT_COLS, H, seqs);
+    if (lanes != 0 && lanes != 16 && lanes != 64) return tli_fail("lightning: 16 or 64 lanes a column, not %d", lanes);
+    if (lanes == 0) lanes = (dk > 32 && (long long)seqs * H * dv < 8LL * 4 * tli_compute_units()) ? 64 : 16;
+    const int cols = LT_THREADS / lanes;
+    const dim3 grid((dv + cols - 1) / cols, H, seqs);
     hipStream_t s = (hipStream_t)stream;
-    const int need = (dk + 15) / 16;
-#define LT_LAUNCH(T, R, CH)                                                                                             \
-    hipLaunchKernelGGL((lightning_recurrence_kernel<T, R, CH>), grid, dim3(LT_THREADS), 0, s, (const T*)proj, ld, decay, \
+    const int need = (dk + lanes - 1) / lanes;
+#define LT_LAUNCH(T, L, R, CH)                                                                                             \
+    hipLaunchKernelGGL((lightning_recurrence_kernel<T, L, R, CH>), grid, dim3(LT_THREADS), 0, s, (const T*)proj, ld, decay, \
                        state, out, row_start, seq_start, slots, H, dk, dv)
-#define LT_SIZES(T)                      \
-    if (need <= 1) LT_LAUNCH(T, 1, 32);  \
-    else if (need <= 2) LT_LAUNCH(T, 2, 32); \
-    else if (need <= 4) LT_LAUNCH(T, 4, 32); \
-    else if (need <= 8) LT_LAUNCH(T, 8, 32); \
-    else LT_LAUNCH(T, 16, 16)
+#define LT_SIZES(T)                                  \
+    if (lanes == 64) {                               \
+        if (need <= 1) LT_LAUNCH(T, 64, 1, 32);      \
+        else if (need <= 2) LT_LAUNCH(T, 64, 2, 32); \
+        else LT_LAUNCH(T, 64, 4, 16);                \
+    } else if (need <= 1) LT_LAUNCH(T, 16, 1, 32);   \
+    else if (need <= 2) LT_LAUNCH(T, 16, 2, 32);     \
+    else if (need <= 4) LT_LAUNCH(T, 16, 4, 32);     \
+    else if (need <= 8) LT_LAUNCH(T, 16, 8, 32);     \
+    else LT_LAUNCH(T, 16, 16, 16)
     if (dtype == TLI_F32) { LT_SIZES(float); }
     else if (dtype == TLI_BF16) { LT_SIZES(bf16_t); }
     else return tli_fail("lightning: unknown dtype %d", dtype);

@@ -128,7 +128,7 @@ def load_library():
         "tli_moe_grouped_bf16": [P, P, P, P, P, P, P, P, P, P, P, P, P, P, P, I, I, I, I, I, I, F, F, P],
         "tli_keyed_prepare": [P, I, P, P, P, P, P, P, P, I, I, I, I, I, I, I, I, P, P, I, I, I, P],
         "tli_add_bias": [P, P, I, I, I, P],
-        "tli_lightning_recurrence": [P, I, P, P, P, P, P, P, I, I, I, I, I, P],
+        "tli_lightning_recurrence": [P, I, P, P, P, P, P, P, I, I, I, I, I, I, P],
         "tli_lightning_norm": [P, P, I, P, P, I, I, F, I, P],
         "tli_sample": [P, I, I, P, P, P, P, P, P],
         "tli_sample_scratch_bytes": [I],
@@ -222,6 +222,7 @@ class HipOps:
         self.attention_tile_rows = 16   # measurements, tests: 32 = tiles of 32 rows in the biased attention kernel (heads up to 128)
         self.moe_tile = 0            # measurements, tests: force the slots of a tile of the routed experts' products (16, 32, 64, 128)
         self.rows_cfg = 0            # measurements: force a launch shape and the k ranges of gemm_rows
+        self.lightning_lanes = 0     # measurements, tests: 16 or 64 lanes a column of the lightning recurrence's state (0: the launch rule)
         self.rows_splits = 0
 
     @property
@@ -1534,7 +1535,7 @@ class HipOps:
         out = torch.empty((T, heads * dv), dtype=torch.float32, device=self.device)
         self._call(self.lib.tli_lightning_recurrence, proj.data_ptr(), proj.shape[1], decay.data_ptr(), state.data_ptr(),
                    out.data_ptr(), step.row_start.data_ptr(), step.seq_start.data_ptr(), step.slots.data_ptr(),
-                   step.num_seqs, heads, dk, dv, _dtype_code(proj.dtype), self._stream())
+                   step.num_seqs, heads, dk, dv, _dtype_code(proj.dtype), int(self.lightning_lanes), self._stream())
         return out
 
     def lightning_norm(self, o, proj, gate_at, weight, eps, out_dtype):
