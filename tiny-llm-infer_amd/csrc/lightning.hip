@@ -12,8 +12,11 @@
 // sequence's rows in order; a column belongs to the 16 lanes of a DPP row (a workgroup then has 16 columns), or to
 // the 64 lanes of a wave (4 columns), lane s holding elements s R .. s R + R - 1 of it in registers (R = dk / lanes
 // rounded up to a power of two; elements from dk on stay zero).  A row costs R multiply-adds for the state, R for
-// the output and four DPP moves (and two exchanges of rows of lanes, with 64 lanes a column).  The rows come through LDS in chunks that the
-// whole workgroup fetches into registers while the chunk before is walked (the silu is taken on their way into LDS).
+// the output and four DPP moves (and two exchanges of rows of lanes, with 64 lanes a column).
+//
+// Two launches: lightning_prepare takes the silu of every row's q, k and v once and leaves them in float32 in a padded
+// layout; lightning_recurrence brings them through LDS in chunks of rows, 16 bytes a copy, which the whole workgroup
+// fetches into registers while the chunk before is walked.
 //
 // lightning_norm: y = o / sqrt(mean(o^2) + eps) * w * sigmoid(gate) over all heads of a row together.
 #include "common.h"
@@ -32,18 +35,41 @@ __device__ __forceinline__ float lt_sum16(float v) {
     return v;
 }
 
+// q, k and v of every row and head with the silu taken, in float32 and in the padded layout that the recurrence
+// stages with 16-byte copies: qk [T][H][2][DKP] (zeros from dk on), v [T][H][DVP] (zeros from dv on)
+template <typename T>
+__global__ void lightning_prepare_kernel(const T* __restrict__ proj, int ld, float* __restrict__ qk, float* __restrict__ v,
+                                         int H, int dk, int dv, int DKP, int DVP) {
+    const size_t row = blockIdx.x;
+    const int h = blockIdx.y;
+    const T* src = proj + row * ld;
+    float* qk_dst = qk + (row * H + h) * 2 * DKP;
+    float* v_dst = v + (row * H + h) * DVP;
+    for (int e = threadIdx.x; e < 2 * DKP + DVP; e += blockDim.x) {
+        if (e < 2 * DKP) {
+            const int i = e < DKP ? e : e - DKP;
+            const size_t at = (e < DKP ? 0 : (size_t)H * dk) + (size_t)h * dk + i;
+            qk_dst[e] = i < dk ? lt_silu(to_f32(src[at])) : 0.f;
+        } else {
+            const int jj = e - 2 * DKP;
+            v_dst[jj] = jj < dv ? lt_silu(to_f32(src[(size_t)2 * H * dk + (size_t)h * dv + jj])) : 0.f;
+        }
+    }
+}
+
 // L lanes a column (16 or 64), R elements of it a lane, CH rows a chunk
-template <typename T, int L, int R, int CH>
+template <int L, int R, int CH>
 __global__ __launch_bounds__(LT_THREADS) void lightning_recurrence_kernel(
-    const T* __restrict__ proj, int ld, const float* __restrict__ decay, float* __restrict__ state,
-    float* __restrict__ out, const int* __restrict__ row_start, const int* __restrict__ seq_start,
-    const int* __restrict__ slots, int H, int dk, int dv) {
+    const float* __restrict__ qk, const float* __restrict__ vals, int DVP, const float* __restrict__ decay,
+    float* __restrict__ state, float* __restrict__ out, const int* __restrict__ row_start,
+    const int* __restrict__ seq_start, const int* __restrict__ slots, int H, int dk, int dv) {
     constexpr int DKP = L * R;
     constexpr int NC = LT_THREADS / L;                   // columns a workgroup
-    constexpr int W = 2 * DKP + 16;                      // floats of a staged row: q, k, the workgroup's values (up to 16)
-    constexpr int PF = CH * W / LT_THREADS;
+    constexpr int W = 2 * DKP + NC;                      // floats of a staged row: q, k, the workgroup's values
+    constexpr int PQ = CH * 2 * DKP / 4 / LT_THREADS;    // 16-byte pieces of q and k that a thread brings a chunk
+    constexpr int PV = CH * NC / 4;                      // pieces of v a chunk, one a thread for the first threads
     constexpr int VW = R % 4 == 0 ? 4 : R % 2 == 0 ? 2 : 1;   // floats a piece of the state that a lane moves at once
-    static_assert(PF * LT_THREADS == CH * W && PF <= 64 && NC <= 16, "a chunk is shared out evenly");
+    static_assert(PQ * LT_THREADS * 4 == CH * 2 * DKP && PV <= LT_THREADS, "a chunk is shared out evenly");
     __shared__ __align__(16) float rows_s[CH * W];
     const int seq = blockIdx.z, h = blockIdx.y, j0 = blockIdx.x * NC;
     const int tid = threadIdx.x;
@@ -77,25 +103,23 @@ __global__ __launch_bounds__(LT_THREADS) void lightning_recurrence_kernel(
                 if (sub * R + r < dk) S[r] = col[sub * R + r];
         }
     }
-    const size_t q_at = (size_t)h * dk, k_at = (size_t)H * dk + (size_t)h * dk, v_at = (size_t)2 * H * dk + (size_t)h * dv;
-    // A chunk's elements are fetched as they lie in memory, every load issued before any is used: which element a
-    // thread takes (its row of the chunk, its column of q, k or v) is arithmetic on constants; an element that does
-    // not exist (past the sequence's end, past dk or dv) is not loaded (where none of a wave's exist, the wave leaves
-    // the load out) or dropped when the chunk is written into LDS, where the silu is taken too.
-    T raw[PF];
-    unsigned long long live = 0;
+    // A chunk is fetched into registers, every load issued before any is used, while the chunk before is walked:
+    // piece p of q and k is 4 floats of row p / (2 DKP / 4) of the chunk; rows past the sequence's end are zeros.
+    const float* qk_seq = qk + ((size_t)r0 * H + h) * 2 * DKP;
+    const float* v_seq = vals + ((size_t)r0 * H + h) * DVP + j0;
+    float4 pq[PQ], pv;
     auto fetch = [&](int first) {
-        live = 0;
 #pragma unroll
-        for (int u = 0; u < PF; ++u) {
-            const int e = tid + u * LT_THREADS;
-            const int rr = e / W, cc = e - rr * W;
-            const int i = cc < DKP ? cc : cc - DKP, jc = cc - 2 * DKP;
-            const size_t at = cc < DKP ? q_at + i : cc < 2 * DKP ? k_at + i : v_at + j0 + jc;
-            const bool ok = first + rr < n && (cc < 2 * DKP ? i < dk : (jc < NC && j0 + jc < dv));
-            raw[u] = 0;
-            if (__builtin_amdgcn_ballot_w64(ok)) raw[u] = proj[ok ? (size_t)(r0 + first + rr) * ld + at : (size_t)r0 * ld + q_at];
-            live |= (unsigned long long)ok << u;
+        for (int u = 0; u < PQ; ++u) {
+            const int p = tid + u * LT_THREADS;
+            const int rr = p / (2 * DKP / 4), c4 = p - rr * (2 * DKP / 4);
+            pq[u] = make_float4(0.f, 0.f, 0.f, 0.f);
+            if (first + rr < n) pq[u] = *reinterpret_cast<const float4*>(qk_seq + (size_t)(first + rr) * H * 2 * DKP + c4 * 4);
+        }
+        pv = make_float4(0.f, 0.f, 0.f, 0.f);
+        if (tid < PV) {
+            const int rr = tid / (NC / 4), c4 = tid - rr * (NC / 4);
+            if (first + rr < n) pv = *reinterpret_cast<const float4*>(v_seq + (size_t)(first + rr) * H * DVP + c4 * 4);
         }
     };
     fetch(0);
@@ -103,7 +127,15 @@ __global__ __launch_bounds__(LT_THREADS) void lightning_recurrence_kernel(
     for (int t0 = 0; t0 < n; t0 += CH) {
         __syncthreads();                                 // the chunk before has been walked by every wave
 #pragma unroll
-        for (int u = 0; u < PF; ++u) rows_s[tid + u * LT_THREADS] = (live >> u & 1) ? lt_silu(to_f32(raw[u])) : 0.f;
+        for (int u = 0; u < PQ; ++u) {
+            const int p = tid + u * LT_THREADS;
+            const int rr = p / (2 * DKP / 4), c4 = p - rr * (2 * DKP / 4);
+            *reinterpret_cast<float4*>(rows_s + rr * W + c4 * 4) = pq[u];
+        }
+        if (tid < PV) {
+            const int rr = tid / (NC / 4), c4 = tid - rr * (NC / 4);
+            *reinterpret_cast<float4*>(rows_s + rr * W + 2 * DKP + c4 * 4) = pv;
+        }
         __syncthreads();
         if (t0 + CH < n) fetch(t0 + CH);
         const int cnt = min(CH, n - t0);
@@ -137,42 +169,71 @@ __global__ __launch_bounds__(LT_THREADS) void lightning_recurrence_kernel(
     }
 }
 
+static int lt_pow2_at_least(int n) {
+    int p = 1;
+    while (p < n) p *= 2;
+    return p;
+}
+
+// How many lanes hold a column of the state (16 or 64; `lanes` 0: 64 where the sequences, heads and columns are too few
+// to give every SIMD of the chip two waves at 16 (one long prompt), else 16: a wave then has four columns and a quarter
+// of the additions across lanes a column), and the padded key size DKP of that layout.
+static int lt_plan(int seqs, int H, int dk, int dv, int lanes, int* dkp) {
+    if (lanes == 0) lanes = (dk > 32 && (long long)seqs * H * dv < 8LL * 4 * tli_compute_units()) ? 64 : 16;
+    *dkp = lanes * lt_pow2_at_least((dk + lanes - 1) / lanes);
+    return lanes;
+}
+
+// float32 elements of scratch that tli_lightning_recurrence wants for `rows` rows
+extern "C" long long tli_lightning_scratch_floats(int rows, int H, int dk, int dv) {
+    int a = 0, b = 0;
+    lt_plan(1, H, dk, dv, 16, &a);
+    lt_plan(1, H, dk, dv, 64, &b);
+    return (long long)rows * H * (2LL * (a > b ? a : b) + (dv + 15) / 16 * 16);
+}
+
 // proj: [T, ld] raw projections, q (H dk), k (H dk), v (H dv) first; decay: float32 [H]; state: float32
-// [slots, H, dv, dk]; out: float32 [T, H dv]; row_start [seqs + 1], seq_start, slots [seqs].
-// lanes: 16 or 64 lanes a column, or 0: 64 where the sequences, heads and columns are too few to give every SIMD of
-// the chip two waves at 16 (one long prompt), else 16 (a wave then has four columns and a quarter of the additions
-// across lanes a column)
+// [slots, H, dv, dk]; out: float32 [T, H dv]; row_start [seqs + 1], seq_start, slots [seqs]; scratch: float32,
+// tli_lightning_scratch_floats(T, ...) elements; lanes: 16 or 64 lanes a column, or 0 for the launch rule
 extern "C" int tli_lightning_recurrence(const void* proj, int ld, const float* decay, float* state, float* out,
-                                        const int* row_start, const int* seq_start, const int* slots, int seqs, int H,
-                                        int dk, int dv, int dtype, int lanes, void* stream) {
-    if (seqs <= 0) return 0;
+                                        float* scratch, const int* row_start, const int* seq_start, const int* slots,
+                                        int T, int seqs, int H, int dk, int dv, int dtype, int lanes, void* stream) {
+    if (seqs <= 0 || T <= 0) return 0;
     if (H <= 0 || dk <= 0 || dv <= 0 || dk > LT_MAX_DK)
         return tli_fail("lightning: bad sizes (heads %d, keys of %d (at most %d), values of %d)", H, dk, LT_MAX_DK, dv);
     if (ld < 2 * H * dk + H * dv) return tli_fail("lightning: rows of %d hold fewer than q, k and v", ld);
     if (H > 65535 || seqs > 65535) return tli_fail("lightning: too many heads or sequences for one launch");
     if (lanes != 0 && lanes != 16 && lanes != 64) return tli_fail("lightning: 16 or 64 lanes a column, not %d", lanes);
-    if (lanes == 0) lanes = (dk > 32 && (long long)seqs * H * dv < 8LL * 4 * tli_compute_units()) ? 64 : 16;
+    if (((uintptr_t)scratch | (uintptr_t)state) & 15) return tli_fail("lightning: scratch and state must be 16-byte aligned");
+    int DKP = 0;
+    lanes = lt_plan(seqs, H, dk, dv, lanes, &DKP);
+    const int DVP = (dv + 15) / 16 * 16;
+    float* qk = scratch;
+    float* vals = scratch + (size_t)T * H * 2 * DKP;
+    hipStream_t s = (hipStream_t)stream;
+    if (dtype == TLI_F32)
+        hipLaunchKernelGGL((lightning_prepare_kernel<float>), dim3(T, H), dim3(256), 0, s, (const float*)proj, ld, qk, vals, H, dk,
+                           dv, DKP, DVP);
+    else if (dtype == TLI_BF16)
+        hipLaunchKernelGGL((lightning_prepare_kernel<bf16_t>), dim3(T, H), dim3(256), 0, s, (const bf16_t*)proj, ld, qk, vals, H,
+                           dk, dv, DKP, DVP);
+    else
+        return tli_fail("lightning: unknown dtype %d", dtype);
     const int cols = LT_THREADS / lanes;
     const dim3 grid((dv + cols - 1) / cols, H, seqs);
-    hipStream_t s = (hipStream_t)stream;
-    const int need = (dk + lanes - 1) / lanes;
-#define LT_LAUNCH(T, L, R, CH)                                                                                             \
-    hipLaunchKernelGGL((lightning_recurrence_kernel<T, L, R, CH>), grid, dim3(LT_THREADS), 0, s, (const T*)proj, ld, decay, \
+    const int R = DKP / lanes;
+#define LT_LAUNCH(L, R, CH)                                                                                         \
+    hipLaunchKernelGGL((lightning_recurrence_kernel<L, R, CH>), grid, dim3(LT_THREADS), 0, s, qk, vals, DVP, decay, \
                        state, out, row_start, seq_start, slots, H, dk, dv)
-#define LT_SIZES(T)                                  \
-    if (lanes == 64) {                               \
-        if (need <= 1) LT_LAUNCH(T, 64, 1, 32);      \
-        else if (need <= 2) LT_LAUNCH(T, 64, 2, 32); \
-        else LT_LAUNCH(T, 64, 4, 16);                \
-    } else if (need <= 1) LT_LAUNCH(T, 16, 1, 32);   \
-    else if (need <= 2) LT_LAUNCH(T, 16, 2, 32);     \
-    else if (need <= 4) LT_LAUNCH(T, 16, 4, 32);     \
-    else if (need <= 8) LT_LAUNCH(T, 16, 8, 32);     \
-    else LT_LAUNCH(T, 16, 16, 16)
-    if (dtype == TLI_F32) { LT_SIZES(float); }
-    else if (dtype == TLI_BF16) { LT_SIZES(bf16_t); }
-    else return tli_fail("lightning: unknown dtype %d", dtype);
-#undef LT_SIZES
+    if (lanes == 64) {
+        if (R == 1) LT_LAUNCH(64, 1, 32);
+        else if (R == 2) LT_LAUNCH(64, 2, 32);
+        else LT_LAUNCH(64, 4, 16);
+    } else if (R == 1) LT_LAUNCH(16, 1, 32);
+    else if (R == 2) LT_LAUNCH(16, 2, 32);
+    else if (R == 4) LT_LAUNCH(16, 4, 32);
+    else if (R == 8) LT_LAUNCH(16, 8, 32);
+    else LT_LAUNCH(16, 16, 16);
 #undef LT_LAUNCH
     return tli_check_launch("lightning_recurrence");
 }

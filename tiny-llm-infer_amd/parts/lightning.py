@@ -62,7 +62,8 @@ class LightningAttention(Mixer):
         return StateNeed(tuple(self.env.ops.lightning_state_shape(self.heads, self.dk, self.dv)), torch.float32)
 
     def workspace_elems(self, rows: int) -> int:
-        return rows * (2 * self.qk_dim + 2 * self.v_dim + 2 * self.v_dim + self.v_dim)
+        # the projections, then q, k, v (padded at worst to twice their size) and o in float32 (two elements of the run's type each at worst)
+        return rows * (2 * self.qk_dim + 2 * self.v_dim + 2 * (4 * self.qk_dim + 2 * self.v_dim) + 2 * self.v_dim + self.v_dim)
 
     def forward(self, x: torch.Tensor, step: StepView):
         ops = self.env.ops
