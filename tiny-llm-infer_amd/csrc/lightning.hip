@@ -175,11 +175,12 @@ static int lt_pow2_at_least(int n) {
     return p;
 }
 
-// How many lanes hold a column of the state (16 or 64; `lanes` 0: 64 where the sequences, heads and columns are too few
-// to give every SIMD of the chip two waves at 16 (one long prompt), else 16: a wave then has four columns and a quarter
-// of the additions across lanes a column), and the padded key size DKP of that layout.
+// How many lanes hold a column of the state (`lanes` 0: 16, where a wave has four columns and a quarter of the additions
+// across lanes a column; 64 lanes a column give one long prompt four times the waves, and were measured level with 16
+// at 16 heads of 128 x 128 and a third slower at 32 heads and in decode steps), and the padded key size DKP of that layout.
 static int lt_plan(int seqs, int H, int dk, int dv, int lanes, int* dkp) {
-    if (lanes == 0) lanes = (dk > 32 && (long long)seqs * H * dv < 8LL * 4 * tli_compute_units()) ? 64 : 16;
+    (void)seqs, (void)H, (void)dv;
+    if (lanes == 0) lanes = 16;
     *dkp = lanes * lt_pow2_at_least((dk + lanes - 1) / lanes);
     return lanes;
 }

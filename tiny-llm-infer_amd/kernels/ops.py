@@ -9,6 +9,7 @@ from __future__ import annotations
 
 import contextlib
 import ctypes
+import os
 from ctypes import c_float, c_int, c_void_p
 from typing import Optional, Tuple
 
@@ -224,7 +225,7 @@ class HipOps:
         self.attention_tile_rows = 16   # measurements, tests: 32 = tiles of 32 rows in the biased attention kernel (heads up to 128)
         self.moe_tile = 0            # measurements, tests: force the slots of a tile of the routed experts' products (16, 32, 64, 128)
         self.rows_cfg = 0            # measurements: force a launch shape and the k ranges of gemm_rows
-        self.lightning_lanes = 0     # measurements, tests: 16 or 64 lanes a column of the lightning recurrence's state (0: the launch rule)
+        self.lightning_lanes = int(os.environ.get("TLI_LIGHTNING_LANES", "0"))   # measurements, tests: 16 or 64 lanes a column of the lightning recurrence's state (0: the launch rule)
         self.rows_splits = 0
 
     @property
