@@ -80,6 +80,16 @@ __device__ __forceinline__ void tile_init(Tile<NJ, ND>& t) {
 template <int NJ, int ND>
 __device__ __forceinline__ float tile_sum(const Tile<NJ, ND>& t) { return t.ls[0] + t.l; }
 
+// What a column's accumulators are multiplied with when it is stored: 1 / (sum of its weights), the sum also holding
+// exp(sink) where the head has a sink.  The weights are exp2(score - base) with the column's base t.m, so the sink's
+// is exp2(sink log2(e) - base); a sink so far above the base that this overflows leaves a factor of 0, its limit.
+template <int NJ, int ND>
+__device__ __forceinline__ float tile_inverse_sum(const Tile<NJ, ND>& t, const float* __restrict__ sinks, int head) {
+    float l = tile_sum(t);
+    if (sinks) l += __builtin_amdgcn_exp2f(sinks[head] * 1.4426950408889634f - t.m);      // (log2(e): scores are kept in units of log2)
+    return l > 0.f ? 1.0f / l : 0.f;
+}
+
 // Load the query of this lane's column: dims [c*8*NJ + 8j, +8) for j < NJ.
 template <int NJ, int ND>
 __device__ __forceinline__ void tile_load_q(Tile<NJ, ND>& t, const bf16_t* q_head, int head_dim, bool live) {
@@ -421,6 +431,9 @@ struct RawQkv {
     const float* partial_sums;
     int parts;
     size_t part_stride;
+    // the prefill kernels only: one logit a query head that stands in the softmax's denominator with no key and
+    // no value (a sink), or null
+    const float* sinks;
 };
 
 // One head of the raw projections as a B operand of the score MFMAs (this lane: dims
@@ -1092,7 +1105,7 @@ attention_prefill_kernel(const bf16_t* __restrict__ q, bf16_t* __restrict__ out,
                          const int* __restrict__ row_start, const int* __restrict__ seq_start,
                          int num_seqs, const int* __restrict__ tables, int table_width, int page_size,
                          int page_shift, int num_pages, int heads, int kv_heads, int head_dim,
-                         float scale, int window, int rq) {
+                         float scale, int window, int rq, const float* __restrict__ sinks) {
     const int lane = threadIdx.x % 64, wave = threadIdx.x / 64, r = lane % 16, c = lane / 16;
     const int group = heads / kv_heads;
     const int head_tiles = (group + 15) / 16;
@@ -1134,8 +1147,7 @@ attention_prefill_kernel(const bf16_t* __restrict__ q, bf16_t* __restrict__ out,
 #pragma unroll
     for (int ct = 0; ct < CT; ++ct) {
         if (!live[ct]) continue;
-        const float l = tile_sum(t[ct]);
-        const float inv = l > 0.f ? 1.0f / l : 0.f;
+        const float inv = tile_inverse_sum(t[ct], sinks, head);
         bf16_t* o = out + ((size_t)row[ct] * heads + head) * head_dim;
 #pragma unroll
         for (int dt = 0; dt < ND; ++dt) {
@@ -1327,8 +1339,7 @@ __device__ __forceinline__ void prefill_lds_block(
 #pragma unroll
     for (int ct = 0; ct < CT; ++ct) {
         if (!live[ct]) continue;
-        const float l = tile_sum(t[ct]);
-        const float inv = l > 0.f ? 1.0f / l : 0.f;
+        const float inv = tile_inverse_sum(t[ct], raw.sinks, head);
         bf16_t* o = out + ((size_t)row[ct] * heads + head) * HD;
 #pragma unroll
         for (int dt = 0; dt < ND; ++dt) {
@@ -1649,14 +1660,14 @@ __device__ __forceinline__ void prefill_pipe_block(
             }
             t[ct].ls = (f32x4){l, l, l, l};
             t[ct].l = 0.f;
+            t[ct].m = base;
         }
     }
 
 #pragma unroll
     for (int ct = 0; ct < CT; ++ct) {
         if (!live[ct]) continue;
-        const float l = tile_sum(t[ct]);
-        const float inv = l > 0.f ? 1.0f / l : 0.f;
+        const float inv = tile_inverse_sum(t[ct], raw.sinks, head);
         bf16_t* o = out + ((size_t)row[ct] * heads + head) * HD;
 #pragma unroll
         for (int dt = 0; dt < ND; ++dt) {
@@ -1903,7 +1914,7 @@ static int launch_prefill(
     const void* q, void* out, const void* k_cache, const void* v_cache, const int* row_start,
     const int* seq_start, int num_seqs, int rows, const int* tables, int table_width, int page_size,
     int num_pages, int heads, int kv_heads, int head_dim, float scale, int window, int direct,
-    const RawQkv* raw_in, void* stream) {
+    const RawQkv* raw_in, const float* sinks, void* stream) {
     if (rows <= 0 || num_seqs <= 0) return 0;
     if (check_common("attention_prefill", heads, kv_heads, head_dim, page_size, table_width, num_pages)) return 1;
     hipStream_t s = (hipStream_t)stream;
@@ -1913,7 +1924,8 @@ static int launch_prefill(
     if (raw_in && (head_dim % 64 || page_size < 8 || direct == 1))
         return tli_fail("attention_prefill from raw projections: head_dim %d must be a multiple of 64, pages "
                         "of at least 8 (%d), through LDS", head_dim, page_size);
-    const RawQkv raw = raw_in ? *raw_in : RawQkv{};
+    RawQkv raw = raw_in ? *raw_in : RawQkv{};
+    raw.sinks = sinks;
     if (page_size >= 8 && direct != 1) {
         // through LDS.  Two column tiles a wave when that still gives two workgroups for every
         // compute unit (long row blocks then come first); else one tile a wave.
@@ -1961,7 +1973,7 @@ static int launch_prefill(
                                : ((size_t)kb * (head_dim + 8) + (size_t)head_dim * (kb + 8)) * sizeof(bf16_t);
 #define ARGS (const bf16_t*)q, (bf16_t*)out, (const bf16_t*)k_cache, (const bf16_t*)v_cache, row_start, \
              seq_start, num_seqs, tables, table_width, page_size, shift, num_pages, heads, kv_heads
-#define TAIL scale * LOG2E, window, rq
+#define TAIL scale * LOG2E, window, rq, sinks
 #define TAIL_LDS scale * LOG2E, window, rq, pair, raw
 #define LDS_CALL(NJ, ND, CT, KB, DMA) attention_prefill_lds_kernel<NJ, ND, CT, KB, DMA><<<grid, 256, lds, s>>>(ARGS, TAIL_LDS)
         if (sets) {
@@ -2011,13 +2023,14 @@ static int launch_prefill(
     return tli_check_launch("attention_prefill");
 }
 
+// sinks: float32 [heads] or null: a logit a query head that the softmax's denominator also holds
 extern "C" int tli_attention_prefill_bf16(
     const void* q, void* out, const void* k_cache, const void* v_cache, const int* row_start,
     const int* seq_start, int num_seqs, int rows, const int* tables, int table_width, int page_size,
     int num_pages, int heads, int kv_heads, int head_dim, float scale, int window, int direct,
-    void* stream) {
+    const float* sinks, void* stream) {
     return launch_prefill(q, out, k_cache, v_cache, row_start, seq_start, num_seqs, rows, tables, table_width,
-                          page_size, num_pages, heads, kv_heads, head_dim, scale, window, direct, nullptr, stream);
+                          page_size, num_pages, heads, kv_heads, head_dim, scale, window, direct, nullptr, sinks, stream);
 }
 
 // The same with the queries taken from the raw projections qkv [rows][(heads + 2 kv_heads) * head_dim]
@@ -2033,5 +2046,5 @@ extern "C" int tli_qkv_attention_prefill_bf16(
     const RawQkv raw{(const bf16_t*)qkv, q_norm_w, nullptr, cos_table, sin_table, q_eps, 0.f, 0};
     return launch_prefill(nullptr, out, k_cache, v_cache, row_start, seq_start, num_seqs, rows, tables,
                           table_width, page_size, num_pages, heads, kv_heads, head_dim, scale, window, direct,
-                          &raw, stream);
+                          &raw, nullptr, stream);
 }

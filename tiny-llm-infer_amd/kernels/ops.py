@@ -93,7 +93,7 @@ def load_library():
         "tli_attention_decode_bf16": [P, P, P, P, P, P, P, P, I, I, I, I, I, I, I, F, I, I, I, P],
         "tli_qkv_attention_decode_bf16": [P, P, P, P, P, P, P, P, I, I, I, I, I, I, I, P, F, P, F, P, P, I,
                                           F, I, I, I, P, I, P],
-        "tli_attention_prefill_bf16": [P, P, P, P, P, P, I, I, P, I, I, I, I, I, I, F, I, I, P],
+        "tli_attention_prefill_bf16": [P, P, P, P, P, P, I, I, P, I, I, I, I, I, I, F, I, I, P, P],
         "tli_qkv_attention_prefill_bf16": [P, P, P, P, P, P, I, I, P, I, I, I, I, I, I, P, F, P, P, F, I, I, P],
         "tli_embed_scaled": [P, P, P, P, P, I, I, I, I, F, I, P],
         "tli_activation": [P, P, ctypes.c_longlong, I, I, P],
@@ -679,8 +679,13 @@ class HipOps:
         if (step.max_seq_len + g.page_size - 1) // g.page_size > g.table_width:
             raise KernelError("a block table is narrower than its sequence needs")
 
-    def paged_attention(self, q, step, cache, heads, kv_heads, head_dim, scale, window):
+    def paged_attention(self, q, step, cache, heads, kv_heads, head_dim, scale, window, sinks=None):
+        """Attention of ``q`` [T, heads * head_dim] over the cache.  ``sinks`` (float32 [heads]): a logit a head that the
+        softmax's denominator also holds; only steps with portions of prompts in bfloat16 take them here (see
+        ``takes_sinks``), everything else goes through ``sized_attention``."""
         T = step.num_rows
+        if sinks is not None and not self.takes_sinks(q.dtype, step, cache, head_dim):
+            raise KernelError("this step's attention kernel has no sink; sized_attention has")
         self._want(q, "queries", None, (T, heads * head_dim))
         if cache is None:
             raise KernelError("attention needs a cache layer")
@@ -693,7 +698,7 @@ class HipOps:
             self._call(self.lib.tli_attention_prefill_bf16, q.data_ptr(), out.data_ptr(), kc.data_ptr(),
                        vc.data_ptr(), step.row_start.data_ptr(), step.seq_start.data_ptr(), step.num_seqs,
                        T, g.tables.data_ptr(), g.table_width, g.page_size, kc.shape[0], heads, kv_heads,
-                       head_dim, float(scale), int(window or 0), self._prefill_mode(step, T),
+                       head_dim, float(scale), int(window or 0), self._prefill_mode(step, T), _ptr(sinks),
                        self._stream())
             return out
         self._call(self.lib.tli_attention_plain, q.data_ptr(), out.data_ptr(), kc.data_ptr(),
@@ -701,6 +706,11 @@ class HipOps:
                    g.tables.data_ptr(), g.table_width, g.page_size, kc.shape[0], T, heads, kv_heads,
                    head_dim, float(scale), int(window or 0), _dtype_code(q.dtype), self._stream())
         return out
+
+    def takes_sinks(self, dtype, step, cache, head_dim) -> bool:
+        """Whether ``paged_attention`` runs this step through the kernel for portions of prompts, which takes sinks."""
+        return (dtype == torch.bfloat16 and head_dim % 16 == 0 and 16 <= head_dim <= 256 and cache.group.page_size >= 4
+                and not self.force_plain and not (step.max_rows_per_seq == 1 and cache.group.page_size >= 8))
 
     def qkv_attention(self, qkv, step, cache, heads, kv_heads, head_dim, q_norm, k_norm, rotary, scale, window):
         """From the raw projections to the attention output: norms and rotation of q
@@ -1498,6 +1508,10 @@ class HipOps:
                    step.positions.data_ptr(), step.seq_of_row.data_ptr(), g.tables.data_ptr(), g.table_width, g.page_size,
                    kc.shape[0], T, heads, kv_heads, head_dim, -1 if values_are_keys else (heads + kv_heads) * head_dim,
                    _ptr(cos), _ptr(sin), rd, npos, _dtype_code(proj.dtype), self._stream())
+        if self.takes_sinks(proj.dtype, step, cache, head_dim):
+            # portions of prompts: the kernel that the stock attention runs them through (keys and values through LDS)
+            return self.paged_attention(q.view(T, heads * head_dim), step, cache, heads, kv_heads, head_dim, scale, window,
+                                        sinks=sinks)
         o = self.sized_attention(q, step, g, kc, vc, heads, kv_heads, 1, head_dim, head_dim, scale, window, 0, proj.dtype,
                                  sinks=sinks)
         return o.view(T, heads * head_dim)
