@@ -189,6 +189,41 @@ def test_lightning_recurrence_in_portions_and_slots_that_are_used_again(ops, dty
             _close(state[slots[i]].transpose(1, 2), final, 2e-5, f"state of sequence {i}")
 
 
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+@pytest.mark.parametrize("heads, dk, dv", [(2, 64, 32), (1, 128, 128), (3, 20, 12)])
+def test_lightning_long_portions_walked_in_segments(ops, dtype, heads, dk, dv):
+    """Portions of hundreds of rows are cut into segments that are walked side by side and joined afterwards: two
+    steps of three sequences (900 + 650, 300 + 1, 5 + 700 rows), the second from the states that the first left, beside
+    a short sequence that is not cut."""
+    g = torch.Generator().manual_seed(dk + dv)
+    dt = DTYPES[dtype]
+    decay = torch.tensor([1.0, 0.99, 0.9][:heads])
+    m = {"heads": heads, "dim": dk, "vdim": dv, "decay": decay.tolist()}
+    width = 2 * heads * dk + 2 * heads * dv
+    eye = torch.eye(width, dtype=F64)
+    names = {"q": eye[:heads * dk], "k": eye[heads * dk:2 * heads * dk], "v": eye[2 * heads * dk:2 * heads * dk + heads * dv],
+             "g": eye[2 * heads * dk + heads * dv:], "o": torch.eye(heads * dv, dtype=F64), "norm": torch.ones(heads * dv, dtype=F64)}
+    state = torch.full((3, *ops.lightning_state_shape(heads, dk, dv)), -3.0, device="cuda")
+    steps = [[900, 300, 5], [650, 1, 700]]
+    proj = [(torch.randn(sum(c), width, generator=g) * 0.5).to(dt) for c in zip(*steps)]
+    got, at = [[], [], []], [0, 0, 0]
+    for counts in steps:
+        rows = torch.cat([proj[i][at[i]:at[i] + c] for i, c in enumerate(counts)]).cuda()
+        view = _view(at, counts, [1, 2, 0])
+        o = ops.lightning_attention(rows, decay.cuda(), state, view, heads, dk, dv)
+        y = ops.lightning_norm(o, rows, 2 * heads * dk + heads * dv, torch.ones(heads * dv, device="cuda"), 1e-5, dt)
+        r = 0
+        for i, c in enumerate(counts):
+            got[i].append(y[r:r + c].cpu())
+            r += c
+            at[i] += c
+    for i in range(3):
+        final = torch.zeros(heads, dk, dv, dtype=F64)
+        want = plain_defosun.lightning(proj[i].double(), m, names, "", 1e-5, state=final)
+        _close(torch.cat(got[i]), want, 2e-5 if dtype == "float32" else 1.5e-2, f"sequence {i}")
+        _close(state[[1, 2, 0][i]].transpose(1, 2), final, 2e-5, f"state of sequence {i}")
+
+
 # ------------------------------------------------------- one mixer alone, every cut ---
 MIXERS = {
     # grouped heads whose values are their keys: sizes in and out of sixteens, all and part of a head turned

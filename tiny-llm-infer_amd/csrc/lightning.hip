@@ -10,8 +10,8 @@
 //
 // Columns of S are independent.  A workgroup takes a few columns of one head of one sequence and walks the
 // sequence's rows in order; a column belongs to the 16 lanes of a DPP row (a workgroup then has 16 columns), or to
-// the 64 lanes of a wave (4 columns), lane s holding elements s R .. s R + R - 1 of it in registers (R = dk / lanes
-// rounded up to a power of two; elements from dk on stay zero).  A row costs R multiply-adds for the state, R for
+// the 64 lanes of a wave (4 columns), a lane holding R elements of it in registers, in pieces of up to four that lie
+// side by side with the other lanes' (R = dk / lanes rounded up to a power of two; elements from dk on stay zero).  A row costs R multiply-adds for the state, R for
 // the output and four DPP moves (and two exchanges of rows of lanes, with 64 lanes a column).
 //
 // Two launches: lightning_prepare takes the silu of every row's q, k and v once and leaves them in float32 in a padded
@@ -57,54 +57,109 @@ __global__ void lightning_prepare_kernel(const T* __restrict__ proj, int ld, flo
     }
 }
 
-// L lanes a column (16 or 64), R elements of it a lane, CH rows a chunk
-template <int L, int R, int CH>
+// A long portion of a prompt is cut into segments of LT_SEGMENT rows that are walked side by side (`seg_rows` > 0):
+// every segment but a portion's first starts from a state of zero and leaves its end state in `carry`; a second
+// launch adds the end states up along the portion (P_1 = E_0, P_(s+1) = c^rows(s) P_s + E_s: what segment s + 1 should
+// have started from; the last sum is the sequence's new state); a third adds to every row of segment s >= 1 what the
+// state it should have started from contributes, c^(t + 1) P_s^T q_t for the segment's row t.  The sums are the
+// recurrence's own, in another order.
+#define LT_SEGMENT 256
+
+struct LtSegment {
+    int seq, first, rows, index, count;                  // the sequence; the first row (within the step's rows of the
+};                                                       // sequence) and the rows; which of how many segments
+
+// segment z of the step, counted sequence by sequence (seg_rows 0: every sequence is one segment); false past the last
+__device__ __forceinline__ bool lt_segment_of(int z, const int* __restrict__ row_start, int num_seqs, int seg_rows,
+                                              LtSegment& s) {
+    if (seg_rows <= 0) {
+        if (z >= num_seqs) return false;
+        s.seq = z, s.first = 0, s.rows = row_start[z + 1] - row_start[z], s.index = 0, s.count = 1;
+        return true;
+    }
+    int before = 0;
+    for (int i = 0; i < num_seqs; ++i) {
+        const int n = row_start[i + 1] - row_start[i];
+        const int c = max(1, (n + seg_rows - 1) / seg_rows);
+        if (z < before + c) {
+            s.seq = i, s.index = z - before, s.count = c, s.first = s.index * seg_rows;
+            s.rows = min(seg_rows, n - s.first);
+            return true;
+        }
+        before += c;
+    }
+    return false;
+}
+
+// L lanes a column (16 or 64), R elements of it a lane, CH rows a chunk.  APPLY: the third launch of a step with
+// segments (the state is the one a segment should have started from and stays as it is; a row's sum is added to
+// what the first launch left in `out`).
+template <int L, int R, int CH, bool APPLY>
 __global__ __launch_bounds__(LT_THREADS) void lightning_recurrence_kernel(
     const float* __restrict__ qk, const float* __restrict__ vals, int DVP, const float* __restrict__ decay,
     float* __restrict__ state, float* __restrict__ out, const int* __restrict__ row_start,
-    const int* __restrict__ seq_start, const int* __restrict__ slots, int H, int dk, int dv) {
+    const int* __restrict__ seq_start, const int* __restrict__ slots, int H, int dk, int dv, int num_seqs, int seg_rows,
+    float* __restrict__ carry) {
     constexpr int DKP = L * R;
     constexpr int NC = LT_THREADS / L;                   // columns a workgroup
     constexpr int W = 2 * DKP + NC;                      // floats of a staged row: q, k, the workgroup's values
     constexpr int PQ = CH * 2 * DKP / 4 / LT_THREADS;    // 16-byte pieces of q and k that a thread brings a chunk
     constexpr int PV = CH * NC / 4;                      // pieces of v a chunk, one a thread for the first threads
-    constexpr int VW = R % 4 == 0 ? 4 : R % 2 == 0 ? 2 : 1;   // floats a piece of the state that a lane moves at once
+    constexpr int VW = R % 4 == 0 ? 4 : R % 2 == 0 ? 2 : 1;   // floats of a piece: what a lane reads or writes at once
     static_assert(PQ * LT_THREADS * 4 == CH * 2 * DKP && PV <= LT_THREADS, "a chunk is shared out evenly");
     __shared__ __align__(16) float rows_s[CH * W];
-    const int seq = blockIdx.z, h = blockIdx.y, j0 = blockIdx.x * NC;
+    __shared__ float power_s[APPLY ? LT_SEGMENT : 1];    // c^(t + 1) for the segment's rows
+    __shared__ float add_s[APPLY ? LT_SEGMENT * NC : 1]; // what the segment's rows get added, [row][column]
+    const int h = blockIdx.y, j0 = blockIdx.x * NC;
     const int tid = threadIdx.x;
     const int sub = tid % L, jl = tid / L;
     const int j = j0 + jl;
-    const int r0 = row_start[seq], n = row_start[seq + 1] - r0;
+    // Element r of a lane is element at(r) of the column: the lanes' pieces of VW floats lie side by side (piece p of
+    // lane s at (p L + s) VW), so that what the column's lanes read from LDS or from the state in one instruction is
+    // one run of memory, which no two of them find in the same bank.
+    auto at = [&](int r) { return (r / VW) * (L * VW) + sub * VW + r % VW; };
+    LtSegment seg;
+    if (!lt_segment_of(blockIdx.z, row_start, num_seqs, seg_rows, seg)) return;      // (the grid's slack)
+    if (APPLY && (seg.count == 1 || seg.index == 0)) return;
+    const int seq = seg.seq, n = seg.rows;
+    const int r0 = row_start[seq] + seg.first;
     if (n <= 0) return;
     const float lam = decay[h];
-    float* col = state + (((size_t)slots[seq] * H + h) * dv + (j < dv ? j : 0)) * dk;
+    // where the state comes from and goes to: the sequence's slot, or the segment's place in `carry`
+    const size_t column = ((size_t)h * dv + (j < dv ? j : 0)) * dk;
+    float* slot_col = state + (size_t)slots[seq] * H * dv * dk + column;
+    float* carry_col = carry + (size_t)blockIdx.z * H * dv * dk + column;
+    const float* from = APPLY ? carry_col : slot_col;
+    const bool read = APPLY || (seg.index == 0 && seq_start[seq] != 0);
+    float* to = seg.count == 1 ? slot_col : carry_col;
     const bool whole = dk == DKP && dk % 4 == 0;         // every lane's elements exist, and its pieces are aligned
     float S[R];
 #pragma unroll
     for (int r = 0; r < R; ++r) S[r] = 0.f;
-    if (seq_start[seq] != 0 && j < dv) {
+    if (read && j < dv) {
         if (whole) {
 #pragma unroll
             for (int r = 0; r < R; r += VW) {
                 if constexpr (VW == 4) {
-                    const float4 v = *reinterpret_cast<const float4*>(col + sub * R + r);
+                    const float4 v = *reinterpret_cast<const float4*>(from + at(r));
                     S[r] = v.x, S[r + 1] = v.y, S[r + 2] = v.z, S[r + 3] = v.w;
                 } else if constexpr (VW == 2) {
-                    const float2 v = *reinterpret_cast<const float2*>(col + sub * R + r);
+                    const float2 v = *reinterpret_cast<const float2*>(from + at(r));
                     S[r] = v.x, S[r + 1] = v.y;
                 } else {
-                    S[r] = col[sub * R + r];
+                    S[r] = from[at(r)];
                 }
             }
         } else {
 #pragma unroll
             for (int r = 0; r < R; ++r)
-                if (sub * R + r < dk) S[r] = col[sub * R + r];
+                if (at(r) < dk) S[r] = from[at(r)];
         }
     }
+    if constexpr (APPLY)
+        for (int t = tid; t < n; t += LT_THREADS) power_s[t] = powf(lam, (float)(t + 1));
     // A chunk is fetched into registers, every load issued before any is used, while the chunk before is walked:
-    // piece p of q and k is 4 floats of row p / (2 DKP / 4) of the chunk; rows past the sequence's end are zeros.
+    // piece p of q and k is 4 floats of row p / (2 DKP / 4) of the chunk; rows past the segment's end are zeros.
     const float* qk_seq = qk + ((size_t)r0 * H + h) * 2 * DKP;
     const float* v_seq = vals + ((size_t)r0 * H + h) * DVP + j0;
     float4 pq[PQ], pv;
@@ -117,7 +172,7 @@ __global__ __launch_bounds__(LT_THREADS) void lightning_recurrence_kernel(
             if (first + rr < n) pq[u] = *reinterpret_cast<const float4*>(qk_seq + (size_t)(first + rr) * H * 2 * DKP + c4 * 4);
         }
         pv = make_float4(0.f, 0.f, 0.f, 0.f);
-        if (tid < PV) {
+        if (!APPLY && tid < PV) {
             const int rr = tid / (NC / 4), c4 = tid - rr * (NC / 4);
             if (first + rr < n) pv = *reinterpret_cast<const float4*>(v_seq + (size_t)(first + rr) * H * DVP + c4 * 4);
         }
@@ -142,31 +197,77 @@ __global__ __launch_bounds__(LT_THREADS) void lightning_recurrence_kernel(
 #pragma unroll 4
         for (int t = 0; t < cnt; ++t) {
             const float* row = rows_s + t * W;
-            const float v = row[2 * DKP + jl];
             float acc = 0.f;
+            if constexpr (APPLY) {
 #pragma unroll
-            for (int r = 0; r < R; ++r) {
-                S[r] = fmaf(lam, S[r], row[DKP + sub * R + r] * v);
-                acc = fmaf(S[r], row[sub * R + r], acc);
+                for (int r = 0; r < R; ++r) acc = fmaf(S[r], row[at(r)], acc);
+            } else {
+                const float v = row[2 * DKP + jl];
+#pragma unroll
+                for (int r = 0; r < R; ++r) {
+                    S[r] = fmaf(lam, S[r], row[DKP + at(r)] * v);
+                    acc = fmaf(S[r], row[at(r)], acc);
+                }
             }
             acc = lt_sum16(acc);
             if constexpr (L == 64) acc = quad_rows_sum(acc);
-            if (sub == 0 && j < dv) o_col[(size_t)(t0 + t) * H * dv] = acc;
+            if constexpr (APPLY) {
+                if (sub == 0) add_s[(t0 + t) * NC + jl] = power_s[t0 + t] * acc;
+            } else if (sub == 0 && j < dv) {
+                o_col[(size_t)(t0 + t) * H * dv] = acc;
+            }
         }
+    }
+    if constexpr (APPLY) {
+        // (added in one go, every load issued before any is used: a row's own read of `out` would be waited for in its turn)
+        __syncthreads();
+        float* o_seg = out + (size_t)r0 * H * dv + (size_t)h * dv + j0;
+        for (int e = tid; e < n * NC; e += LT_THREADS) {
+            const int t = e / NC, c = e - t * NC;
+            if (j0 + c < dv) o_seg[(size_t)t * H * dv + c] += add_s[e];
+        }
+        return;
     }
     if (j >= dv) return;
     if (whole) {
 #pragma unroll
         for (int r = 0; r < R; r += VW) {
-            if constexpr (VW == 4) *reinterpret_cast<float4*>(col + sub * R + r) = make_float4(S[r], S[r + 1], S[r + 2], S[r + 3]);
-            else if constexpr (VW == 2) *reinterpret_cast<float2*>(col + sub * R + r) = make_float2(S[r], S[r + 1]);
-            else col[sub * R + r] = S[r];
+            if constexpr (VW == 4) *reinterpret_cast<float4*>(to + at(r)) = make_float4(S[r], S[r + 1], S[r + 2], S[r + 3]);
+            else if constexpr (VW == 2) *reinterpret_cast<float2*>(to + at(r)) = make_float2(S[r], S[r + 1]);
+            else to[at(r)] = S[r];
         }
     } else {
 #pragma unroll
         for (int r = 0; r < R; ++r)
-            if (sub * R + r < dk) col[sub * R + r] = S[r];
+            if (at(r) < dk) to[at(r)] = S[r];
     }
+}
+
+// The second launch of a step with segments: one thread an element of a sequence's state.  carry[z] holds the end
+// state E of segment z and is left holding the state P that the segment should have started from; the sequence's slot
+// gets its new state.
+__global__ void lightning_carry_kernel(float* __restrict__ carry, float* __restrict__ state, const float* __restrict__ decay,
+                                       const int* __restrict__ row_start, const int* __restrict__ slots, int num_seqs,
+                                       int seg_rows, int H, int dv, int dk) {
+    const int seq = blockIdx.y;
+    const size_t per = (size_t)H * dv * dk;
+    const size_t e = (size_t)blockIdx.x * blockDim.x + threadIdx.x;
+    if (e >= per) return;
+    int z0 = 0;
+    for (int i = 0; i < seq; ++i) z0 += max(1, (row_start[i + 1] - row_start[i] + seg_rows - 1) / seg_rows);
+    const int n = row_start[seq + 1] - row_start[seq];
+    const int count = max(1, (n + seg_rows - 1) / seg_rows);
+    if (count == 1) return;                              // (its one segment wrote the slot itself)
+    const float lam = decay[e / ((size_t)dv * dk)];
+    const float whole = powf(lam, (float)seg_rows), last = powf(lam, (float)(n - (count - 1) * seg_rows));
+    float p = carry[(size_t)z0 * per + e];
+    for (int s = 1; s < count; ++s) {
+        float* at = carry + (size_t)(z0 + s) * per + e;
+        const float end = *at;
+        *at = p;
+        p = fmaf(s == count - 1 ? last : whole, p, end);
+    }
+    state[(size_t)slots[seq] * per + e] = p;
 }
 
 static int lt_pow2_at_least(int n) {
@@ -178,27 +279,35 @@ static int lt_pow2_at_least(int n) {
 // How many lanes hold a column of the state (`lanes` 0: 16, where a wave has four columns and a quarter of the additions
 // across lanes a column; 64 lanes a column give one long prompt four times the waves, and were measured level with 16
 // at 16 heads of 128 x 128 and a third slower at 32 heads and in decode steps), and the padded key size DKP of that layout.
-static int lt_plan(int seqs, int H, int dk, int dv, int lanes, int* dkp) {
-    (void)seqs, (void)H, (void)dv;
+static int lt_plan(int dk, int lanes, int* dkp) {
     if (lanes == 0) lanes = 16;
     *dkp = lanes * lt_pow2_at_least((dk + lanes - 1) / lanes);
     return lanes;
 }
 
-// float32 elements of scratch that tli_lightning_recurrence wants for `rows` rows
-extern "C" long long tli_lightning_scratch_floats(int rows, int H, int dk, int dv) {
+// The rows of a segment, or 0 where the step's portions are walked whole: segments pay from about one and a half of
+// them on (a second and a third launch, and the third walks the rows once more).
+static int lt_segment_rows(int longest) { return longest > LT_SEGMENT + LT_SEGMENT / 2 ? LT_SEGMENT : 0; }
+
+// float32 elements of scratch that tli_lightning_recurrence wants for a step of `rows` rows in `seqs` sequences whose
+// longest portion has `longest` rows
+extern "C" long long tli_lightning_scratch_floats(int rows, int seqs, int longest, int H, int dk, int dv) {
     int a = 0, b = 0;
-    lt_plan(1, H, dk, dv, 16, &a);
-    lt_plan(1, H, dk, dv, 64, &b);
-    return (long long)rows * H * (2LL * (a > b ? a : b) + (dv + 15) / 16 * 16);
+    lt_plan(dk, 16, &a);
+    lt_plan(dk, 64, &b);
+    const int seg = lt_segment_rows(longest);
+    const long long segments = seg ? rows / seg + seqs : 0;
+    return (long long)rows * H * (2LL * (a > b ? a : b) + (dv + 15) / 16 * 16) + segments * H * dv * dk;
 }
 
 // proj: [T, ld] raw projections, q (H dk), k (H dk), v (H dv) first; decay: float32 [H]; state: float32
 // [slots, H, dv, dk]; out: float32 [T, H dv]; row_start [seqs + 1], seq_start, slots [seqs]; scratch: float32,
-// tli_lightning_scratch_floats(T, ...) elements; lanes: 16 or 64 lanes a column, or 0 for the launch rule
+// tli_lightning_scratch_floats(T, ...) elements; longest: the most rows that a sequence brings (an upper bound will do);
+// lanes: 16 or 64 lanes a column, or 0 for the launch rule
 extern "C" int tli_lightning_recurrence(const void* proj, int ld, const float* decay, float* state, float* out,
                                         float* scratch, const int* row_start, const int* seq_start, const int* slots,
-                                        int T, int seqs, int H, int dk, int dv, int dtype, int lanes, void* stream) {
+                                        int T, int seqs, int longest, int H, int dk, int dv, int dtype, int lanes,
+                                        void* stream) {
     if (seqs <= 0 || T <= 0) return 0;
     if (H <= 0 || dk <= 0 || dv <= 0 || dk > LT_MAX_DK)
         return tli_fail("lightning: bad sizes (heads %d, keys of %d (at most %d), values of %d)", H, dk, LT_MAX_DK, dv);
@@ -207,10 +316,14 @@ extern "C" int tli_lightning_recurrence(const void* proj, int ld, const float* d
     if (lanes != 0 && lanes != 16 && lanes != 64) return tli_fail("lightning: 16 or 64 lanes a column, not %d", lanes);
     if (((uintptr_t)scratch | (uintptr_t)state) & 15) return tli_fail("lightning: scratch and state must be 16-byte aligned");
     int DKP = 0;
-    lanes = lt_plan(seqs, H, dk, dv, lanes, &DKP);
+    lanes = lt_plan(dk, lanes, &DKP);
     const int DVP = (dv + 15) / 16 * 16;
     float* qk = scratch;
-    float* vals = scratch + (size_t)T * H * 2 * DKP;
+    float* vals = qk + (size_t)T * H * 2 * DKP;
+    float* carry = vals + (size_t)T * H * DVP;
+    const int seg = lt_segment_rows(longest);
+    const int zs = seg ? T / seg + seqs : seqs;          // (an upper bound of the segments; a workgroup past the last leaves)
+    if (zs > 65535) return tli_fail("lightning: too many segments for one launch");
     hipStream_t s = (hipStream_t)stream;
     if (dtype == TLI_F32)
         hipLaunchKernelGGL((lightning_prepare_kernel<float>), dim3(T, H), dim3(256), 0, s, (const float*)proj, ld, qk, vals, H, dk,
@@ -221,20 +334,29 @@ extern "C" int tli_lightning_recurrence(const void* proj, int ld, const float* d
     else
         return tli_fail("lightning: unknown dtype %d", dtype);
     const int cols = LT_THREADS / lanes;
-    const dim3 grid((dv + cols - 1) / cols, H, seqs);
+    const dim3 grid((dv + cols - 1) / cols, H, zs);
     const int R = DKP / lanes;
-#define LT_LAUNCH(L, R, CH)                                                                                         \
-    hipLaunchKernelGGL((lightning_recurrence_kernel<L, R, CH>), grid, dim3(LT_THREADS), 0, s, qk, vals, DVP, decay, \
-                       state, out, row_start, seq_start, slots, H, dk, dv)
-    if (lanes == 64) {
-        if (R == 1) LT_LAUNCH(64, 1, 32);
-        else if (R == 2) LT_LAUNCH(64, 2, 32);
-        else LT_LAUNCH(64, 4, 16);
-    } else if (R == 1) LT_LAUNCH(16, 1, 32);
-    else if (R == 2) LT_LAUNCH(16, 2, 32);
-    else if (R == 4) LT_LAUNCH(16, 4, 32);
-    else if (R == 8) LT_LAUNCH(16, 8, 32);
-    else LT_LAUNCH(16, 16, 16);
+#define LT_LAUNCH(L, R, CH, APPLY)                                                                                         \
+    hipLaunchKernelGGL((lightning_recurrence_kernel<L, R, CH, APPLY>), grid, dim3(LT_THREADS), 0, s, qk, vals, DVP, decay, \
+                       state, out, row_start, seq_start, slots, H, dk, dv, seqs, seg, carry)
+#define LT_SIZES(APPLY)                                  \
+    if (lanes == 64) {                                   \
+        if (R == 1) LT_LAUNCH(64, 1, 32, APPLY);         \
+        else if (R == 2) LT_LAUNCH(64, 2, 32, APPLY);    \
+        else LT_LAUNCH(64, 4, 16, APPLY);                \
+    } else if (R == 1) LT_LAUNCH(16, 1, 32, APPLY);      \
+    else if (R == 2) LT_LAUNCH(16, 2, 32, APPLY);        \
+    else if (R == 4) LT_LAUNCH(16, 4, 32, APPLY);        \
+    else if (R == 8) LT_LAUNCH(16, 8, 32, APPLY);        \
+    else LT_LAUNCH(16, 16, 16, APPLY)
+    LT_SIZES(false);
+    if (seg) {
+        const size_t per = (size_t)H * dv * dk;
+        hipLaunchKernelGGL(lightning_carry_kernel, dim3((unsigned)((per + 255) / 256), seqs), dim3(256), 0, s, carry, state, decay,
+                           row_start, slots, seqs, seg, H, dv, dk);
+        LT_SIZES(true);
+    }
+#undef LT_SIZES
 #undef LT_LAUNCH
     return tli_check_launch("lightning_recurrence");
 }

@@ -129,7 +129,7 @@ def load_library():
         "tli_moe_grouped_bf16": [P, P, P, P, P, P, P, P, P, P, P, P, P, P, P, I, I, I, I, I, I, F, F, P],
         "tli_keyed_prepare": [P, I, P, P, P, P, P, P, P, I, I, I, I, I, I, I, I, P, P, I, I, I, P],
         "tli_add_bias": [P, P, I, I, I, P],
-        "tli_lightning_recurrence": [P, I, P, P, P, P, P, P, P, I, I, I, I, I, I, I, P],
+        "tli_lightning_recurrence": [P, I, P, P, P, P, P, P, P, I, I, I, I, I, I, I, I, P],
         "tli_lightning_norm": [P, P, I, P, P, I, I, F, I, P],
         "tli_sample": [P, I, I, P, P, P, P, P, P],
         "tli_sample_scratch_bytes": [I],
@@ -139,7 +139,7 @@ def load_library():
         fn = getattr(lib, name)
         fn.argtypes = args
         fn.restype = c_int
-    lib.tli_lightning_scratch_floats.argtypes = [I, I, I, I]
+    lib.tli_lightning_scratch_floats.argtypes = [I, I, I, I, I, I]
     lib.tli_lightning_scratch_floats.restype = ctypes.c_longlong
     lib.tli_sample_uniform.argtypes = [ctypes.c_uint32, ctypes.c_uint32, ctypes.c_uint32]
     lib.tli_sample_uniform.restype = c_float
@@ -1550,12 +1550,15 @@ class HipOps:
         if max(step.h_slots, default=0) >= state.shape[0]:
             raise KernelError("a sequence's slot lies outside the state")
         out = torch.empty((T, heads * dv), dtype=torch.float32, device=self.device)
-        # (silu(q), silu(k), silu(v) of the step in float32, padded as the recurrence's lanes hold them)
-        scratch = torch.empty((int(self.lib.tli_lightning_scratch_floats(T, heads, dk, dv)),), dtype=torch.float32, device=self.device)
+        # (silu(q), silu(k), silu(v) of the step in float32, padded as the recurrence's lanes hold them,
+        # and, where long portions are walked in segments side by side, the segments' states)
+        longest = int(step.max_rows_per_seq)
+        scratch = torch.empty((int(self.lib.tli_lightning_scratch_floats(T, step.num_seqs, longest, heads, dk, dv)),),
+                              dtype=torch.float32, device=self.device)
         self._call(self.lib.tli_lightning_recurrence, proj.data_ptr(), proj.shape[1], decay.data_ptr(), state.data_ptr(),
                    out.data_ptr(), scratch.data_ptr(), step.row_start.data_ptr(), step.seq_start.data_ptr(),
-                   step.slots.data_ptr(), T, step.num_seqs, heads, dk, dv, _dtype_code(proj.dtype), int(self.lightning_lanes),
-                   self._stream())
+                   step.slots.data_ptr(), T, step.num_seqs, longest, heads, dk, dv, _dtype_code(proj.dtype),
+                   int(self.lightning_lanes), self._stream())
         return out
 
     def lightning_norm(self, o, proj, gate_at, weight, eps, out_dtype):
