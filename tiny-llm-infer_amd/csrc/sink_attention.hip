@@ -107,6 +107,23 @@ __global__ void add_bias_kernel(T* __restrict__ y, const float* __restrict__ bia
     from_f32(y + idx, to_f32(y[idx]) + bias[idx % n]);
 }
 
+// eight elements a thread, 16-byte accesses: n % 8 == 0
+__global__ void add_bias_vec_kernel(bf16_t* __restrict__ y, const float* __restrict__ bias, int n, size_t groups) {
+    const size_t g = (size_t)blockIdx.x * blockDim.x + threadIdx.x;
+    if (g >= groups) return;
+    const int col = (int)(g % (n / 8)) * 8;
+    uint4* at = reinterpret_cast<uint4*>(y) + g;
+    const uint4 v = *at;
+    const uint32_t w[4] = {v.x, v.y, v.z, v.w};
+    const float4 b0 = *reinterpret_cast<const float4*>(bias + col), b1 = *reinterpret_cast<const float4*>(bias + col + 4);
+    const float b[8] = {b0.x, b0.y, b0.z, b0.w, b1.x, b1.y, b1.z, b1.w};
+    uint32_t o[4];
+#pragma unroll
+    for (int i = 0; i < 4; ++i)
+        o[i] = pack_bf16x2(bf16_to_f32((bf16_t)(w[i] & 0xffffu)) + b[2 * i], bf16_to_f32((bf16_t)(w[i] >> 16)) + b[2 * i + 1]);
+    *at = make_uint4(o[0], o[1], o[2], o[3]);
+}
+
 // y: [rows, n] in place; bias: float32 [n]
 extern "C" int tli_add_bias(void* y, const float* bias, int rows, int n, int dtype, void* stream) {
     if (rows <= 0) return 0;
@@ -115,6 +132,8 @@ extern "C" int tli_add_bias(void* y, const float* bias, int rows, int n, int dty
     const unsigned blocks = (unsigned)((total + 255) / 256);
     hipStream_t s = (hipStream_t)stream;
     if (dtype == TLI_F32) hipLaunchKernelGGL((add_bias_kernel<float>), dim3(blocks), dim3(256), 0, s, (float*)y, bias, n, total);
+    else if (dtype == TLI_BF16 && n % 8 == 0 && !(((uintptr_t)y | (uintptr_t)bias) & 15))
+        hipLaunchKernelGGL(add_bias_vec_kernel, dim3((unsigned)((total / 8 + 255) / 256)), dim3(256), 0, s, (bf16_t*)y, bias, n, total / 8);
     else if (dtype == TLI_BF16) hipLaunchKernelGGL((add_bias_kernel<bf16_t>), dim3(blocks), dim3(256), 0, s, (bf16_t*)y, bias, n, total);
     else return tli_fail("add_bias: unknown dtype %d", dtype);
     return tli_check_launch("add_bias");
