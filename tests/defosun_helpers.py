@@ -72,7 +72,7 @@ SMALL = {
     # sizes in sixteens (the matrix-core kernels), pages of 32, two streams, the first two layers passed twice
     "R": (_config(320, 128, [_layer("attention", _attention(8, 2, 64, 16, base=100000.0), _R_MOE),
                              _layer("lightning", _lightning(4, 64, 32, [0.8, 0.95, 0.99, 0.999]), _dense(256)),
-                             _layer("latent_attention", _latent(4, 64, 32, 48, 96, base=50000.0), _R_MOE)],
+                             _layer("latent_attention", _latent(4, 64, 32, 48, 80, base=30000.0), _R_MOE)],
                   streams=2, loop=(0, 2, 2)), 32, 7),
 }
 
