@@ -190,7 +190,7 @@ def test_lightning_recurrence_in_portions_and_slots_that_are_used_again(ops, dty
 
 
 @pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
-@pytest.mark.parametrize("heads, dk, dv", [(2, 64, 32), (1, 128, 128), (3, 20, 12)])
+@pytest.mark.parametrize("heads, dk, dv", [(2, 64, 32), (1, 128, 128), (3, 20, 12), (2, 30, 70), (1, 256, 40)])
 def test_lightning_long_portions_walked_in_segments(ops, dtype, heads, dk, dv):
     """Portions of hundreds of rows are cut into segments that are walked side by side and joined afterwards: two
     steps of three sequences (900 + 650, 300 + 1, 5 + 700 rows), the second from the states that the first left, beside

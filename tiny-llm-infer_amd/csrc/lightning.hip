@@ -16,7 +16,8 @@
 //
 // Two launches: lightning_prepare takes the silu of every row's q, k and v once and leaves them in float32 in a padded
 // layout; lightning_recurrence brings them through LDS in chunks of rows, 16 bytes a copy, which the whole workgroup
-// fetches into registers while the chunk before is walked.
+// fetches into registers while the chunk before is walked.  Two more where a portion is long enough to be cut into
+// segments (lightning_carry, lightning_apply: see LT_SEGMENT below).
 //
 // lightning_norm: y = o / sqrt(mean(o^2) + eps) * w * sigmoid(gate) over all heads of a row together.
 #include "common.h"
@@ -60,8 +61,8 @@ __global__ void lightning_prepare_kernel(const T* __restrict__ proj, int ld, flo
 // A long portion of a prompt is cut into segments of LT_SEGMENT rows that are walked side by side (`seg_rows` > 0):
 // every segment but a portion's first starts from a state of zero and leaves its end state in `carry`; a second
 // launch adds the end states up along the portion (P_1 = E_0, P_(s+1) = c^rows(s) P_s + E_s: what segment s + 1 should
-// have started from; the last sum is the sequence's new state); a third adds to every row of segment s >= 1 what the
-// state it should have started from contributes, c^(t + 1) P_s^T q_t for the segment's row t.  The sums are the
+// have started from; the last sum is the sequence's new state); a third (lightning_apply) adds to every row of segment
+// s >= 1 what the state it should have started from contributes, c^(t + 1) P_s^T q_t for the segment's row t.  The sums are the
 // recurrence's own, in another order.
 #define LT_SEGMENT 256
 
@@ -91,10 +92,8 @@ __device__ __forceinline__ bool lt_segment_of(int z, const int* __restrict__ row
     return false;
 }
 
-// L lanes a column (16 or 64), R elements of it a lane, CH rows a chunk.  APPLY: the third launch of a step with
-// segments (the state is the one a segment should have started from and stays as it is; a row's sum is added to
-// what the first launch left in `out`).
-template <int L, int R, int CH, bool APPLY>
+// L lanes a column (16 or 64), R elements of it a lane, CH rows a chunk
+template <int L, int R, int CH>
 __global__ __launch_bounds__(LT_THREADS) void lightning_recurrence_kernel(
     const float* __restrict__ qk, const float* __restrict__ vals, int DVP, const float* __restrict__ decay,
     float* __restrict__ state, float* __restrict__ out, const int* __restrict__ row_start,
@@ -108,8 +107,6 @@ __global__ __launch_bounds__(LT_THREADS) void lightning_recurrence_kernel(
     constexpr int VW = R % 4 == 0 ? 4 : R % 2 == 0 ? 2 : 1;   // floats of a piece: what a lane reads or writes at once
     static_assert(PQ * LT_THREADS * 4 == CH * 2 * DKP && PV <= LT_THREADS, "a chunk is shared out evenly");
     __shared__ __align__(16) float rows_s[CH * W];
-    __shared__ float power_s[APPLY ? LT_SEGMENT : 1];    // c^(t + 1) for the segment's rows
-    __shared__ float add_s[APPLY ? LT_SEGMENT * NC : 1]; // what the segment's rows get added, [row][column]
     const int h = blockIdx.y, j0 = blockIdx.x * NC;
     const int tid = threadIdx.x;
     const int sub = tid % L, jl = tid / L;
@@ -120,7 +117,6 @@ __global__ __launch_bounds__(LT_THREADS) void lightning_recurrence_kernel(
     auto at = [&](int r) { return (r / VW) * (L * VW) + sub * VW + r % VW; };
     LtSegment seg;
     if (!lt_segment_of(blockIdx.z, row_start, num_seqs, seg_rows, seg)) return;      // (the grid's slack)
-    if (APPLY && (seg.count == 1 || seg.index == 0)) return;
     const int seq = seg.seq, n = seg.rows;
     const int r0 = row_start[seq] + seg.first;
     if (n <= 0) return;
@@ -129,8 +125,8 @@ __global__ __launch_bounds__(LT_THREADS) void lightning_recurrence_kernel(
     const size_t column = ((size_t)h * dv + (j < dv ? j : 0)) * dk;
     float* slot_col = state + (size_t)slots[seq] * H * dv * dk + column;
     float* carry_col = carry + (size_t)blockIdx.z * H * dv * dk + column;
-    const float* from = APPLY ? carry_col : slot_col;
-    const bool read = APPLY || (seg.index == 0 && seq_start[seq] != 0);
+    const float* from = slot_col;
+    const bool read = seg.index == 0 && seq_start[seq] != 0;
     float* to = seg.count == 1 ? slot_col : carry_col;
     const bool whole = dk == DKP && dk % 4 == 0;         // every lane's elements exist, and its pieces are aligned
     float S[R];
@@ -156,8 +152,6 @@ __global__ __launch_bounds__(LT_THREADS) void lightning_recurrence_kernel(
                 if (at(r) < dk) S[r] = from[at(r)];
         }
     }
-    if constexpr (APPLY)
-        for (int t = tid; t < n; t += LT_THREADS) power_s[t] = powf(lam, (float)(t + 1));
     // A chunk is fetched into registers, every load issued before any is used, while the chunk before is walked:
     // piece p of q and k is 4 floats of row p / (2 DKP / 4) of the chunk; rows past the segment's end are zeros.
     const float* qk_seq = qk + ((size_t)r0 * H + h) * 2 * DKP;
@@ -172,7 +166,7 @@ __global__ __launch_bounds__(LT_THREADS) void lightning_recurrence_kernel(
             if (first + rr < n) pq[u] = *reinterpret_cast<const float4*>(qk_seq + (size_t)(first + rr) * H * 2 * DKP + c4 * 4);
         }
         pv = make_float4(0.f, 0.f, 0.f, 0.f);
-        if (!APPLY && tid < PV) {
+        if (tid < PV) {
             const int rr = tid / (NC / 4), c4 = tid - rr * (NC / 4);
             if (first + rr < n) pv = *reinterpret_cast<const float4*>(v_seq + (size_t)(first + rr) * H * DVP + c4 * 4);
         }
@@ -197,36 +191,17 @@ __global__ __launch_bounds__(LT_THREADS) void lightning_recurrence_kernel(
 #pragma unroll 4
         for (int t = 0; t < cnt; ++t) {
             const float* row = rows_s + t * W;
+            const float v = row[2 * DKP + jl];
             float acc = 0.f;
-            if constexpr (APPLY) {
 #pragma unroll
-                for (int r = 0; r < R; ++r) acc = fmaf(S[r], row[at(r)], acc);
-            } else {
-                const float v = row[2 * DKP + jl];
-#pragma unroll
-                for (int r = 0; r < R; ++r) {
-                    S[r] = fmaf(lam, S[r], row[DKP + at(r)] * v);
-                    acc = fmaf(S[r], row[at(r)], acc);
-                }
+            for (int r = 0; r < R; ++r) {
+                S[r] = fmaf(lam, S[r], row[DKP + at(r)] * v);
+                acc = fmaf(S[r], row[at(r)], acc);
             }
             acc = lt_sum16(acc);
             if constexpr (L == 64) acc = quad_rows_sum(acc);
-            if constexpr (APPLY) {
-                if (sub == 0) add_s[(t0 + t) * NC + jl] = power_s[t0 + t] * acc;
-            } else if (sub == 0 && j < dv) {
-                o_col[(size_t)(t0 + t) * H * dv] = acc;
-            }
+            if (sub == 0 && j < dv) o_col[(size_t)(t0 + t) * H * dv] = acc;
         }
-    }
-    if constexpr (APPLY) {
-        // (added in one go, every load issued before any is used: a row's own read of `out` would be waited for in its turn)
-        __syncthreads();
-        float* o_seg = out + (size_t)r0 * H * dv + (size_t)h * dv + j0;
-        for (int e = tid; e < n * NC; e += LT_THREADS) {
-            const int t = e / NC, c = e - t * NC;
-            if (j0 + c < dv) o_seg[(size_t)t * H * dv + c] += add_s[e];
-        }
-        return;
     }
     if (j >= dv) return;
     if (whole) {
@@ -268,6 +243,84 @@ __global__ void lightning_carry_kernel(float* __restrict__ carry, float* __restr
         p = fmaf(s == count - 1 ? last : whole, p, end);
     }
     state[(size_t)slots[seq] * per + e] = p;
+}
+
+// The third launch of a step with segments: out[t, :] += c^(t + 1) P^T q_t for the rows t of every segment but a
+// portion's first, P the state that the segment should have started from (left in `carry` by the second launch, a
+// head's [dv][dk]).  A product of float32 matrices: a wave takes 16 rows of a segment and NT tiles of 16 columns (a
+// workgroup 64 rows), and
+// multiplies on the matrix cores with v_mfma_f32_16x16x4_f32, which takes float32 as it is (A: lane l has row l % 16,
+// k = l / 16; B: k = l / 16, column l % 16; the sums: rows 4 (l / 16) .. + 3 of column l % 16).  Of 16 consecutive k,
+// lane group c takes 4 c .. 4 c + 3 in four instructions (the order of k does not matter as long as q and P agree),
+// so that a lane loads its four elements of q, and of P, in one piece of 16 bytes, straight from memory: both were
+// written by the launches before and lie in the cache.
+typedef float lt_f32x4 __attribute__((ext_vector_type(4)));
+
+template <int NT>
+__global__ __launch_bounds__(LT_THREADS) void lightning_apply_kernel(
+    const float* __restrict__ qk, int DKP, const float* __restrict__ decay, float* __restrict__ out,
+    const int* __restrict__ row_start, int H, int dk, int dv, int num_seqs, int seg_rows, const float* __restrict__ carry) {
+    LtSegment seg;
+    if (!lt_segment_of(blockIdx.z, row_start, num_seqs, seg_rows, seg)) return;      // (the grid's slack)
+    if (seg.count == 1 || seg.index == 0) return;
+    // (a workgroup: 64 rows of the segment, 16 a wave, and 16 NT columns; blockIdx.x counts the groups of rows first)
+    constexpr int ROW_GROUPS = LT_SEGMENT / 64;
+    const int h = blockIdx.y, jb = (blockIdx.x / ROW_GROUPS) * 16 * NT;
+    const int lane = threadIdx.x % TLI_WAVE, wave = threadIdx.x / TLI_WAVE, r = lane % 16, c = lane / 16;
+    const int r0 = row_start[seg.seq] + seg.first, n = seg.rows;
+    const float lam = decay[h];
+    const float* P = carry + ((size_t)blockIdx.z * H + h) * dv * dk;
+    const bool whole = dk % 4 == 0;                      // a lane's four elements of a column exist together, aligned
+    const int t0 = (blockIdx.x % ROW_GROUPS) * 64 + wave * 16;
+    if (t0 < n) {
+        const bool live = t0 + r < n;
+        const float* q_row = qk + ((size_t)(r0 + (live ? t0 + r : 0)) * H + h) * 2 * DKP;    // (zeros from dk on)
+        lt_f32x4 acc[NT];
+#pragma unroll
+        for (int nt = 0; nt < NT; ++nt) acc[nt] = (lt_f32x4){0.f, 0.f, 0.f, 0.f};
+#pragma unroll 2
+        for (int kb = 0; kb < DKP; kb += 16) {
+            const int i = kb + 4 * c;
+            float4 a = make_float4(0.f, 0.f, 0.f, 0.f);
+            if (live) a = *reinterpret_cast<const float4*>(q_row + i);
+            float4 b[NT];
+#pragma unroll
+            for (int nt = 0; nt < NT; ++nt) {
+                const int j = jb + nt * 16 + r;
+                b[nt] = make_float4(0.f, 0.f, 0.f, 0.f);
+                if (j < dv && i < dk) {
+                    const float* p = P + (size_t)j * dk + i;
+                    if (whole) {
+                        b[nt] = *reinterpret_cast<const float4*>(p);
+                    } else {
+                        b[nt].x = p[0];
+                        if (i + 1 < dk) b[nt].y = p[1];
+                        if (i + 2 < dk) b[nt].z = p[2];
+                        if (i + 3 < dk) b[nt].w = p[3];
+                    }
+                }
+            }
+#pragma unroll
+            for (int nt = 0; nt < NT; ++nt) {
+                acc[nt] = __builtin_amdgcn_mfma_f32_16x16x4f32(a.x, b[nt].x, acc[nt], 0, 0, 0);
+                acc[nt] = __builtin_amdgcn_mfma_f32_16x16x4f32(a.y, b[nt].y, acc[nt], 0, 0, 0);
+                acc[nt] = __builtin_amdgcn_mfma_f32_16x16x4f32(a.z, b[nt].z, acc[nt], 0, 0, 0);
+                acc[nt] = __builtin_amdgcn_mfma_f32_16x16x4f32(a.w, b[nt].w, acc[nt], 0, 0, 0);
+            }
+        }
+#pragma unroll
+        for (int v = 0; v < 4; ++v) {
+            const int t = t0 + 4 * c + v;
+            if (t >= n) continue;
+            const float power = powf(lam, (float)(t + 1));
+            float* o = out + (size_t)(r0 + t) * H * dv + (size_t)h * dv;
+#pragma unroll
+            for (int nt = 0; nt < NT; ++nt) {
+                const int j = jb + nt * 16 + r;
+                if (j < dv) o[j] += power * acc[nt][v];
+            }
+        }
+    }
 }
 
 static int lt_pow2_at_least(int n) {
@@ -336,28 +389,31 @@ extern "C" int tli_lightning_recurrence(const void* proj, int ld, const float* d
     const int cols = LT_THREADS / lanes;
     const dim3 grid((dv + cols - 1) / cols, H, zs);
     const int R = DKP / lanes;
-#define LT_LAUNCH(L, R, CH, APPLY)                                                                                         \
-    hipLaunchKernelGGL((lightning_recurrence_kernel<L, R, CH, APPLY>), grid, dim3(LT_THREADS), 0, s, qk, vals, DVP, decay, \
+#define LT_LAUNCH(L, R, CH)                                                                                         \
+    hipLaunchKernelGGL((lightning_recurrence_kernel<L, R, CH>), grid, dim3(LT_THREADS), 0, s, qk, vals, DVP, decay, \
                        state, out, row_start, seq_start, slots, H, dk, dv, seqs, seg, carry)
-#define LT_SIZES(APPLY)                                  \
-    if (lanes == 64) {                                   \
-        if (R == 1) LT_LAUNCH(64, 1, 32, APPLY);         \
-        else if (R == 2) LT_LAUNCH(64, 2, 32, APPLY);    \
-        else LT_LAUNCH(64, 4, 16, APPLY);                \
-    } else if (R == 1) LT_LAUNCH(16, 1, 32, APPLY);      \
-    else if (R == 2) LT_LAUNCH(16, 2, 32, APPLY);        \
-    else if (R == 4) LT_LAUNCH(16, 4, 32, APPLY);        \
-    else if (R == 8) LT_LAUNCH(16, 8, 32, APPLY);        \
-    else LT_LAUNCH(16, 16, 16, APPLY)
-    LT_SIZES(false);
+    if (lanes == 64) {
+        if (R == 1) LT_LAUNCH(64, 1, 32);
+        else if (R == 2) LT_LAUNCH(64, 2, 32);
+        else LT_LAUNCH(64, 4, 16);
+    } else if (R == 1) LT_LAUNCH(16, 1, 32);
+    else if (R == 2) LT_LAUNCH(16, 2, 32);
+    else if (R == 4) LT_LAUNCH(16, 4, 32);
+    else if (R == 8) LT_LAUNCH(16, 8, 32);
+    else LT_LAUNCH(16, 16, 16);
+#undef LT_LAUNCH
     if (seg) {
         const size_t per = (size_t)H * dv * dk;
         hipLaunchKernelGGL(lightning_carry_kernel, dim3((unsigned)((per + 255) / 256), seqs), dim3(256), 0, s, carry, state, decay,
                            row_start, slots, seqs, seg, H, dv, dk);
-        LT_SIZES(true);
+        // (four tiles of 16 columns a wave where the head has them: q is then loaded once for 64 columns)
+        if (dv > 32)
+            hipLaunchKernelGGL((lightning_apply_kernel<4>), dim3((dv + 63) / 64 * (LT_SEGMENT / 64), H, zs), dim3(LT_THREADS), 0, s, qk, DKP, decay, out,
+                               row_start, H, dk, dv, seqs, seg, carry);
+        else
+            hipLaunchKernelGGL((lightning_apply_kernel<2>), dim3((dv + 31) / 32 * (LT_SEGMENT / 64), H, zs), dim3(LT_THREADS), 0, s, qk, DKP, decay, out,
+                               row_start, H, dk, dv, seqs, seg, carry);
     }
-#undef LT_SIZES
-#undef LT_LAUNCH
     return tli_check_launch("lightning_recurrence");
 }
 
