@@ -234,6 +234,8 @@ MIXERS = {
     "keys as values 2/1 128 (64 turned)": ("attention", _attention(2, 1, 128, 64, base=1e6)),
     "keys as values 34/2 16 (2 turned)": ("attention", _attention(34, 2, 16, 2)),
     "keys as values 3/3 20 (10 turned)": ("attention", _attention(3, 3, 20, 10)),
+    "keys as values 4/2 48 (24 turned)": ("attention", _attention(4, 2, 48, 24)),
+    "keys as values 5/1 96 (32 turned)": ("attention", _attention(5, 1, 96, 32, base=1e5)),
     # one latent vector a position, the key part turned in pairs of neighbours
     "latent 3 64+16 -> 96 of 80": ("latent_attention", _latent(3, 64, 16, 96, 80, base=1e6)),
     "latent 5 24+6 -> 20 of 40": ("latent_attention", _latent(5, 24, 6, 20, 40)),
@@ -325,8 +327,9 @@ def test_one_key_far_back_and_at_the_borders_of_pages(tmp_path, dtype, page, at)
     _last_token_three_ways(folder, dtype, page, toks, want, f"needle at {at}")
 
 
+@pytest.mark.parametrize("page", [4, 16])
 @pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
-def test_a_sink_that_takes_most_of_the_weight(tmp_path, dtype):
+def test_a_sink_that_takes_most_of_the_weight(tmp_path, dtype, page):
     """With a sink far above every score the heads give next to nothing; with one far below, the softmax is the plain one;
     a kernel that left the sink out, scaled it, or counted it a key at a time would show in either."""
     logits = {}
@@ -335,7 +338,7 @@ def test_a_sink_that_takes_most_of_the_weight(tmp_path, dtype):
         w = plain_defosun.read_model(folder)[1]
         toks = [t % 88 for t in random_prompt(88, 150, 3)]
         logits[sink] = plain_defosun.forward(cfg, w, toks)[-1].numpy()
-        _last_token_three_ways(folder, dtype, 16, toks, logits[sink], f"sink {sink}")
+        _last_token_three_ways(folder, dtype, page, toks, logits[sink], f"sink {sink}")
     assert np.abs(logits[6.0] - logits[-30.0]).max() > 0.04 * np.abs(logits[-30.0]).max()
     assert np.abs(logits[12.0] - logits[6.0]).max() > 0.04 * np.abs(logits[6.0]).max()
 
