@@ -225,6 +225,7 @@ class HipOps:
         self.attention_tile_rows = 16   # measurements, tests: 32 = tiles of 32 rows in the biased attention kernel (heads up to 128)
         self.moe_tile = 0            # measurements, tests: force the slots of a tile of the routed experts' products (16, 32, 64, 128)
         self.rows_cfg = 0            # measurements: force a launch shape and the k ranges of gemm_rows
+        self.sinks_in_prefill = os.environ.get("TLI_SINKS_IN_PREFILL", "1") != "0"   # measurements, tests: False sends portions of prompts with sinks through sized_attention too
         self.lightning_lanes = int(os.environ.get("TLI_LIGHTNING_LANES", "0"))   # measurements, tests: 16 or 64 lanes a column of the lightning recurrence's state (0: the launch rule)
         self.rows_splits = 0
 
@@ -709,8 +710,8 @@ class HipOps:
 
     def takes_sinks(self, dtype, step, cache, head_dim) -> bool:
         """Whether ``paged_attention`` runs this step through the kernel for portions of prompts, which takes sinks."""
-        return (dtype == torch.bfloat16 and head_dim % 16 == 0 and 16 <= head_dim <= 256 and cache.group.page_size >= 4
-                and not self.force_plain and not (step.max_rows_per_seq == 1 and cache.group.page_size >= 8))
+        return (self.sinks_in_prefill and dtype == torch.bfloat16 and head_dim % 16 == 0 and 16 <= head_dim <= 256
+                and cache.group.page_size >= 4 and not self.force_plain and not (step.max_rows_per_seq == 1 and cache.group.page_size >= 8))
 
     def qkv_attention(self, qkv, step, cache, heads, kv_heads, head_dim, q_norm, k_norm, rotary, scale, window):
         """From the raw projections to the attention output: norms and rotation of q
